@@ -23,7 +23,7 @@ def _library():
     tail = [F, P, I, I, I, I, I, I, I, I, I, I, F, P]     # eps .. stream
     lib.tff_attention_decode_fused.argtypes = [P, I, P, P, P, P, P, P, I, P, P, P, P, P] + tail
     lib.tff_attention_decode_fused_static.argtypes = [P, I, P, P, P, P, I, P, P, P, P, P] + tail
-    lib.tff_attention_split_reduce.argtypes = [P, P, P, I, I, I, I, P, I, P]
+    lib.tff_attention_split_reduce.argtypes = [P, P, P, I, I, I, I, P, I, P, P]
     for f in (lib.tff_attention_decode_fused, lib.tff_attention_decode_fused_static, lib.tff_attention_split_reduce):
         f.restype = I
     return lib
@@ -82,7 +82,7 @@ def _run(lib, t, splits, static):
         assert rc == 0, lib.tff_last_error().decode()
         if splits > 1:
             rc = lib.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R, nq,
-                                                d, None, 0, None)
+                                                d, None, 0, None, None)
             assert rc == 0, lib.tff_last_error().decode()
     torch.cuda.synchronize()
     return out, k, v

@@ -7,7 +7,7 @@
 //                                              reference paged_flash_attention.cu:723)
 //   visible iff  lo <= j <= pos               (causal: mask_op.cu:37-43; lo from the window)
 //   running max m and sum l over chunks       (paged_flash_attention.cu:746-790)
-//   o = sum_j exp(s_j - m) v_j / l
+//   o = sum_j exp(s_j - m) v_j / l            (l also holds e^(sink - m) of the head, if sinks are given)
 // q head h reads kv head h / (nq / nkv)       (paged_flash_attention.cu:891-892).
 // Keys lie [page, kv head, slot, element], values [page, kv head, element, slot].
 // Keys are found by block id arithmetic, not by a table of addresses as in the
@@ -22,7 +22,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, const TC* __restrict__ k_cache,
     const TC* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
     const int32_t* __restrict__ token_req, const int32_t* __restrict__ positions, int nq, int nkv,
-    int d, int page_size, int window, float scale) {
+    int d, int page_size, int window, float scale, const float* __restrict__ sinks) {
     __shared__ float qs[AG_MAX_D];
     __shared__ long long voff[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -79,6 +79,8 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         }
     }
     T* op = out + (size_t)t * nq * d + (size_t)h * d;
+    // a sink: one more term e^sink in the denominator, with no key and no value, not scaled
+    if (sinks) l += expf(sinks[h] - m);
     const float inv = 1.0f / l;
 #pragma unroll
     for (int i = 0; i < AG_MAX_D / 64; ++i) {
@@ -91,7 +93,8 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out, const 
                                   const void* v_cache, const int32_t* block_tables, int bt_stride,
                                   const int32_t* token_req, const int32_t* positions, int T, int nq,
                                   int nkv, int d, int page_size, int num_pages, int window,
-                                  float scale, int dtype, int cache_dtype, tff_stream_t stream) {
+                                  float scale, const float* sinks, int dtype, int cache_dtype,
+                                  tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && token_req && positions,
                 "attention: null pointer");
     TFF_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
@@ -110,12 +113,12 @@ TFF_API int tff_attention_generic(const void* q, int q_stride, void* out, const 
     if (dtype == TFF_F32)
         attention_generic_kernel<float, float><<<grid, 64, 0, s>>>(
             (const float*)q, q_stride, (float*)out, (const float*)k_cache, (const float*)v_cache,
-            block_tables, bt_stride, token_req, positions, nq, nkv, d, page_size, window, scale);
+            block_tables, bt_stride, token_req, positions, nq, nkv, d, page_size, window, scale, sinks);
     else if (dtype == TFF_BF16)
         attention_generic_kernel<bf16_t, bf16_t><<<grid, 64, 0, s>>>(
             (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache,
             (const bf16_t*)v_cache, block_tables, bt_stride, token_req, positions, nq, nkv, d,
-            page_size, window, scale);
+            page_size, window, scale, sinks);
     else
         return tff_fail("attention: unknown dtype %d", dtype);
     return tff_check_launch("attention_generic");

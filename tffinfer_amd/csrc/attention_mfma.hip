@@ -77,6 +77,10 @@ struct AttnFuse {
     // (entry, first key, end of keys, the entry's position), 16 bytes, and gets a wave per kv head.
     // An entry of negative number: the run is not in use.
     const int32_t* key_runs;
+    // One number per query head that stands in the softmax's denominator beside the keys' terms,
+    // e^sink, with no key and no value: not scaled, counted once however the keys are split
+    // (the kernel or merge that forms the final sum adds it).  Null: none.
+    const float* sinks;
 };
 
 // RMS norm over the head and rotation of one head held as MFMA operand fragments: lane group kg
@@ -553,6 +557,7 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
             wgt[w] = ms == -INFINITY ? 0.f : __expf(ms - m);
             lsum = fmaf(mml[w * 32 + qc * 2 + 1], wgt[w], lsum);
         }
+        if (fz.sinks && !run_is_partial) lsum += __expf(fz.sinks[c_head] - m);
         const float inv = 1.0f / lsum;
         bf16_t* op = out + ((size_t)c_tok * nq + c_head) * D;
         // (a run of an entry that has several: the block's result is a partial one, kept by run)
@@ -599,6 +604,7 @@ __global__ __launch_bounds__(64 * BW, 1) void attn_wave_kernel(
             part_ml[row * 2 + 1] = l;
         }
     } else {
+        if (fz.sinks) l += __expf(fz.sinks[c_head] - m_run * scale);
         const float inv = 1.0f / l;
         bf16_t* op = out + ((size_t)c_tok * nq + c_head) * D;
 #pragma unroll
@@ -617,7 +623,8 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
                                                                  const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, int splits,
                                                                  int R_total, int nq, int d,
-                                                                 const int32_t* __restrict__ rows) {
+                                                                 const int32_t* __restrict__ rows,
+                                                                 const float* __restrict__ sinks) {
     __shared__ float w[256];
     __shared__ float red[17];
     // rows: (entry, token) pairs; without them entry i is token i
@@ -649,7 +656,7 @@ __global__ __launch_bounds__(256) void attn_split_reduce_kernel(const float* __r
     }
     const float l = block_sum(ls * ws, red);   // its barriers also publish w and used_w
     const int used = max(max(used_w[0], used_w[1]), max(used_w[2], used_w[3]));
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / (sinks ? l + __expf(sinks[h] - m) : l);
     for (int e = tid; e < d; e += blockDim.x) {
         float acc = 0.f;
         int s0 = 0;
@@ -674,7 +681,8 @@ __global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float*
                                                                  const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, int splits,
                                                                  int R_total, int nq, int d,
-                                                                 const int32_t* __restrict__ rows, int n) {
+                                                                 const int32_t* __restrict__ rows, int n,
+                                                                 const float* __restrict__ sinks) {
     const int lane = threadIdx.x & 63;
     const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);     // (row, head), heads fastest
     if (pair >= n * nq) return;
@@ -704,6 +712,7 @@ __global__ __launch_bounds__(256) void attn_split_reduce_few_kernel(const float*
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = fmaf(v[u][e], w[u], acc[e]);
     }
+    if (sinks) l += __expf(sinks[h] - m);
     const float inv = 1.0f / l;
     bf16_t* o = out + ((size_t)t * nq + h) * d;
 #pragma unroll
@@ -726,7 +735,8 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
                                                               bf16_t* __restrict__ out,
                                                               const int32_t* __restrict__ run_start,
                                                               const int32_t* __restrict__ tokens,
-                                                              int R, int nq, int d) {
+                                                              int R, int nq, int d,
+                                                              const float* __restrict__ sinks) {
     constexpr int AHEAD = 16;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int pair = blockIdx.x;                              // (entry, head), heads fastest
@@ -805,6 +815,7 @@ __global__ __launch_bounds__(256) void attn_run_merge_kernel(const float* __rest
             l += sum_l[o];
         }
     }
+    if (sinks) l += __expf(sinks[h] - m);
     const float inv = 1.0f / l;
     bf16_t* o = out + ((size_t)(tokens ? tokens[r] : r) * nq + h) * d;   // (tokens: the row of out that entry r's token has)
     if (e0 < d) {
@@ -847,7 +858,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
     const int32_t* __restrict__ block_tables, int bt_stride, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ start_pos, const int32_t* __restrict__ work,
     const int32_t* __restrict__ block_items, int nq, int nkv, int page_size, int page_shift,
-    int window, float scale) {
+    int window, float scale, const float* __restrict__ sinks) {
     constexpr int D = DT * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KFR = 2 * KS, VFR = DT, FR = KFR + VFR;   // 1 KB fragments per slice
@@ -1148,6 +1159,7 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
             const float a1 = m_run[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run[t] - m) * sl2);
             const float a2 = m2 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m2 - m) * sl2);
             l_run[t] = l_run[t] * a1 + l2 * a2;
+            m_run[t] = m;      // (what the sum is relative to from here on: the sink's term needs it)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const float4 o2 = *reinterpret_cast<const float4*>(mt + dt * 256 + lane * 4);
@@ -1164,6 +1176,8 @@ __global__ __launch_bounds__(64 * NW * KGRP, (NW * KGRP <= 4 ? 2 : 1)) void attn
         float l = l_run[t];
         l = rows_sum(l);
         if (!c_ok[t]) continue;
+        // (the sink's term e^(sink - m), with the reference m = m_run * scale as the keys' terms have it)
+        if (sinks) l += __builtin_amdgcn_exp2f(fmaf(sinks[c_head[t]], 1.4426950408889634f, -m_run[t] * sl2));
         const float inv = 1.0f / l;
         bf16_t* op = out + ((size_t)c_tok[t] * nq + c_head[t]) * D;
 #pragma unroll
@@ -1185,7 +1199,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
                        int tiles_per_entry, int cols_per_wave,
                        int splits, int nq, int nkv, int page_size, int window, float scale,
                        int T_total, hipStream_t s, const AttnFuse* fuse = nullptr, int key_groups = 2,
-                       const AttnFuse* runs_only = nullptr) {
+                       const AttnFuse* runs_only = nullptr, const float* sinks = nullptr) {
     int page_shift = 0;   // the page size is a power of two (tff_attention_mfma_supported)
     while ((1 << page_shift) < page_size) ++page_shift;
     if (cols_per_wave == 256) {
@@ -1195,7 +1209,7 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
         if constexpr (DT <= 8) {
             attn_mfma_block_kernel<DT, 2, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                 q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale);
+                block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
             return tff_check_launch("attention_mfma_block256");
         } else {
             return tff_fail("attention_mfma: blocks of 256 columns take head sizes up to 128");
@@ -1210,21 +1224,22 @@ static int launch_attn(const bf16_t* q, int q_stride, bf16_t* out, float* part_o
             if (key_groups == 2)
                 attn_mfma_block_kernel<DT, 1, 8, 2><<<dim3(num_blocks, nkv), 1024, 0, s>>>(
                     q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                    block_items, nq, nkv, page_size, page_shift, window, scale);
+                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
             else
                 attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                     q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                    block_items, nq, nkv, page_size, page_shift, window, scale);
+                    block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
         } else
             attn_mfma_block_kernel<DT, 1, 8, 1><<<dim3(num_blocks, nkv), 512, 0, s>>>(
                 q, q_stride, out, k_cache, v_cache, block_tables, bt_stride, cu_tokens, start_pos, work,
-                block_items, nq, nkv, page_size, page_shift, window, scale);
+                block_items, nq, nkv, page_size, page_shift, window, scale, sinks);
         return tff_check_launch("attention_mfma_block");
     }
     const dim3 grid(num_work, nkv, max(splits, 1));
     // (runs_only: nothing to fuse, q is finished and the pages hold the tokens; only the runs of keys are set)
-    const AttnFuse fz = fuse ? *fuse : runs_only ? *runs_only
-                                                 : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr};
+    AttnFuse fz = fuse ? *fuse : runs_only ? *runs_only
+                                           : AttnFuse{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, nullptr, nullptr};
+    if (sinks) fz.sinks = sinks;
 #define TFF_ATTN_ARGS                                                                              \
     q, q_stride, out, part_o, part_ml, k_cache, v_cache, block_tables, bt_stride, cu_tokens,       \
         start_pos, work, tiles_per_entry, nq, nkv, page_size, page_shift, window, scale, T_total
@@ -1276,7 +1291,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
-                               float scale, tff_stream_t stream) {
+                               float scale, const float* sinks, tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
                 "attention_mfma: null pointer");
     TFF_REQUIRE(key_groups == 1 || key_groups == 2, "attention_mfma: %d key groups (1 or 2)", key_groups);
@@ -1318,7 +1333,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                 bt_stride, cu_tokens, start_pos, work, num_work, block_items,       \
                                 num_blocks, tiles_per_entry,                                        \
                                 cols_per_wave, splits, nq, nkv, page_size, window, scale, T_total, s, \
-                                nullptr, key_groups);
+                                nullptr, key_groups, nullptr, splits > 1 ? nullptr : sinks);
     switch (d) {
         TFF_ATTN_CASE(1) TFF_ATTN_CASE(2) TFF_ATTN_CASE(3) TFF_ATTN_CASE(4) TFF_ATTN_CASE(5)
         TFF_ATTN_CASE(6) TFF_ATTN_CASE(7) TFF_ATTN_CASE(8) TFF_ATTN_CASE(12) TFF_ATTN_CASE(16)
@@ -1388,7 +1403,7 @@ TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* ou
 
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
                                        int splits, int R_total, int nq, int d, const int32_t* rows,
-                                       int num_rows, tff_stream_t stream) {
+                                       int num_rows, const float* sinks, tff_stream_t stream) {
     TFF_REQUIRE(part_o && part_ml && out, "attention_split_reduce: null pointer");
     TFF_REQUIRE(splits >= 1 && R_total >= 0 && nq > 0 && nq <= 65535 && d > 0,
                 "attention_split_reduce: bad sizes");
@@ -1398,10 +1413,10 @@ TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml
     TFF_REQUIRE(splits <= 256, "attention_split_reduce: at most 256 splits, got %d", splits);
     if (splits <= 4 && d <= 256)
         attn_split_reduce_few_kernel<<<(n * nq + 3) / 4, 256, 0, (hipStream_t)stream>>>(
-            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows, n);
+            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows, n, sinks);
     else
         attn_split_reduce_kernel<<<dim3(n, nq), 256, 0, (hipStream_t)stream>>>(
-            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows);
+            part_o, part_ml, (bf16_t*)out, splits, R_total, nq, d, rows, sinks);
     return tff_check_launch("attention_split_reduce");
 }
 
@@ -1472,7 +1487,7 @@ TFF_API int tff_attention_decode_runs(const void* qkv, int qkv_stride, void* out
     }
 #undef TFF_ATTN_CASE
     if (rc || !merge) return rc;
-    attn_run_merge_kernel<<<R * nq, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, nullptr, R, nq, d);
+    attn_run_merge_kernel<<<R * nq, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, nullptr, R, nq, d, nullptr);
     return tff_check_launch("attention_run_merge");
 }
 
@@ -1490,7 +1505,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                                     const int32_t* key_runs, const int32_t* run_start,
                                     const int32_t* tokens, int num_runs, int num_entries, int merge,
                                     int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                    int window, float scale, tff_stream_t stream) {
+                                    int window, float scale, const float* sinks, tff_stream_t stream) {
     TFF_REQUIRE(q && out && k_cache && v_cache && block_tables && cu_tokens && start_pos,
                 "attention_mfma_runs: null pointer");
     TFF_REQUIRE(key_runs && run_start && tokens && part_o && part_ml,
@@ -1509,7 +1524,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                 "65,535), head size %d (at most 256)", num_runs, nkv, tiles, d);
     TFF_REQUIRE(bt_stride > 0 && num_pages > 0 && window >= 0 && num_entries >= 0 && T >= 0, "attention_mfma_runs: bad geometry");
     if (num_entries == 0 || num_runs == 0) return 0;
-    AttnFuse fz{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, key_runs};
+    AttnFuse fz{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0, key_runs, sinks};
     hipStream_t s = (hipStream_t)stream;
     int rc = -1;
 #define TFF_ATTN_CASE(DTV)                                                                          \
@@ -1527,7 +1542,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
 #undef TFF_ATTN_CASE
     if (rc || !merge) return rc;
     attn_run_merge_kernel<<<num_entries * nq, 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, run_start, tokens,
-                                                                    num_entries, nq, d);
+                                                                    num_entries, nq, d, sinks);
     return tff_check_launch("attention_run_merge");
 }
 
@@ -1598,6 +1613,6 @@ TFF_API int tff_attention_decode_fused_static(const void* qkv, int qkv_stride, v
                                             window, scale, stream))
         return rc;
     if (splits > 1 && R > 0)
-        return tff_attention_split_reduce(part_o, part_ml, out, splits, R, nq, d, nullptr, 0, stream);
+        return tff_attention_split_reduce(part_o, part_ml, out, splits, R, nq, d, nullptr, 0, nullptr, stream);
     return 0;
 }

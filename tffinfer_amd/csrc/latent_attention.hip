@@ -1,0 +1,194 @@
+// Latent attention: what stands around the paged attention kernels when keys and values are
+// kept as one low-rank latent vector per token.
+//
+// Per token the cache holds c (kv_rank elements, RMS-normed) and one rotated key part kr
+// (rot elements) that all heads share.  With the up-projections taken to the query's side,
+//   score_h(i, j) = (Wuk_h^T q_h^nope)(i) . c(j) + q_h^rot(i) . kr(j)
+//   out_h(i)      = Wuv_h (sum_j p_h(i, j) c(j))
+// the attention itself is attention with ONE key head of size kv_rank + rot whose values are
+// the first kv_rank elements of its keys, which the paged kernels of this library run as they
+// are: a key page row is [c | kr | 0 ..] up to the padded head size Dp, the (transposed) value
+// page holds c in its first kv_rank rows and zeros below.
+//
+// tff_latent_kv_store:  c = rmsnorm(x[:rank]) * w, kr = rotate(x[rank:]) into the token's slot.
+// tff_head_linear:      out[t, h, :N] = x[t, h, :K] . Wt[h]  (Wt [H, K, N]), per head, with
+//                       an optional sigmoid gate on the result and an optional tail of the
+//                       input row that is rotated by the token's position and copied behind
+//                       the product (the query's rotated part), zeros up to pad_to.
+#include "common.h"
+#include "tffinfer_kernels.h"
+
+template <typename T, typename TC>
+__global__ __launch_bounds__(256) void latent_kv_store_kernel(
+    const T* __restrict__ x, int x_stride, int rank, int rot, int rot_dims,
+    const float* __restrict__ norm_w, float eps, const float* __restrict__ cos_sin, int max_pos,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, TC* __restrict__ k_cache,
+    TC* __restrict__ v_cache, int page_size, int Dp) {
+    __shared__ float red[17];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int slot = slots[t];
+    if (slot < 0) return;      // (the whole block: a token that writes no key)
+    const T* xr = x + (size_t)t * x_stride;
+    float ss = 0.f;
+    for (int e = tid; e < rank; e += blockDim.x) {
+        const float v = to_f32(xr[e]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rr = 1.0f / sqrtf(ss / (float)rank + eps);
+    const int page = slot / page_size, off = slot - page * page_size;
+    TC* kr = k_cache + ((size_t)page * page_size + off) * Dp;
+    TC* vr = v_cache + (size_t)page * Dp * page_size + off;
+    for (int e = tid; e < rank; e += blockDim.x) {
+        const TC c = from_f32<TC>(to_f32(xr[e]) * rr * norm_w[e]);
+        kr[e] = c;
+        vr[(size_t)e * page_size] = c;
+    }
+    int pos = positions[t];
+    pos = min(max(pos, 0), max_pos - 1);
+    const float* cs = cos_sin ? cos_sin + (size_t)pos * rot_dims : nullptr;   // [pair][cos, sin]
+    for (int e = tid; e < Dp - rank; e += blockDim.x) {
+        float v = 0.f;
+        if (e < rot) {
+            v = to_f32(xr[rank + e]);
+            if (cs && e < rot_dims) {
+                const int i = e >> 1;
+                const float c = cs[2 * i], s = cs[2 * i + 1];
+                const float u = to_f32(xr[rank + 2 * i]), w = to_f32(xr[rank + 2 * i + 1]);
+                v = (e & 1) ? fmaf(w, c, u * s) : fmaf(u, c, -(w * s));
+            }
+        }
+        kr[rank + e] = from_f32<TC>(v);
+    }
+}
+
+TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims,
+                                const float* norm_w, float eps, const float* cos_sin, int max_pos,
+                                const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
+                                int page_size, int num_pages, int Dp, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(x && norm_w && positions && slots && k_cache && v_cache, "latent_kv_store: null pointer");
+    TFF_REQUIRE(T >= 0 && rank > 0 && rot >= 0 && Dp >= rank + rot && x_stride >= rank + rot,
+                "latent_kv_store: bad sizes rank=%d rot=%d padded=%d stride=%d", rank, rot, Dp, x_stride);
+    TFF_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && max_pos > 0)),
+                "latent_kv_store: %d rotated dimensions of %d need an even count and a table", rot_dims, rot);
+    TFF_REQUIRE(page_size > 0 && num_pages > 0, "latent_kv_store: bad cache geometry");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TFF_F32)
+        latent_kv_store_kernel<float, float><<<T, 256, 0, s>>>((const float*)x, x_stride, rank, rot, rot_dims, norm_w, eps,
+                                                               rot_dims ? cos_sin : nullptr, max_pos, positions, slots,
+                                                               (float*)k_cache, (float*)v_cache, page_size, Dp);
+    else if (dtype == TFF_BF16)
+        latent_kv_store_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)x, x_stride, rank, rot, rot_dims, norm_w, eps,
+                                                                 rot_dims ? cos_sin : nullptr, max_pos, positions, slots,
+                                                                 (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, Dp);
+    else
+        return tff_fail("latent_kv_store: unknown dtype %d", dtype);
+    return tff_check_launch("latent_kv_store");
+}
+
+// ---------------------------------------------------------------- per-head products ---
+// One block per (TT tokens, head, 256 output columns).  The block's input rows go to LDS as
+// float32, KC elements at a time; thread n walks k, reading Wt[h][k][n] (neighbouring threads,
+// neighbouring addresses) and adding into TT accumulators, k ascending for every token
+// whatever the batch.
+#define HL_TT 8
+#define HL_KC 128
+
+struct HeadLinearTail {
+    int tail;            // elements of the input row behind the K multiplied ones that are copied behind the product
+    int rot_dims;        // of which the first rot_dims are rotated in pairs (2i, 2i+1)
+    int pad_to;          // the output's head is filled with zeros up to this many elements
+    int max_pos;
+    const float* cos_sin;          // [position][pair][cos, sin], rot_dims / 2 pairs
+    const int32_t* positions;      // per token
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_linear_kernel(
+    const T* __restrict__ x, int x_row, int x_head, const T* __restrict__ Wt, T* __restrict__ out, int out_row,
+    int out_head, int Tn, int K, int N, const T* __restrict__ gate, int gate_row, HeadLinearTail tl) {
+    __shared__ float xs[HL_TT][HL_KC];
+    const int t0 = blockIdx.x * HL_TT, h = blockIdx.y, tid = threadIdx.x;
+    const int n = blockIdx.z * 256 + tid;
+    const int nt = min(HL_TT, Tn - t0);
+    const T* W = Wt + (size_t)h * K * N;
+    float acc[HL_TT];
+#pragma unroll
+    for (int i = 0; i < HL_TT; ++i) acc[i] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += HL_KC) {
+        const int kc = min(HL_KC, K - k0);
+        __syncthreads();
+        for (int i = tid; i < HL_TT * HL_KC; i += 256) {
+            const int tt = i / HL_KC, k = i - tt * HL_KC;
+            xs[tt][k] = (tt < nt && k < kc) ? to_f32(x[(size_t)(t0 + tt) * x_row + (size_t)h * x_head + k0 + k]) : 0.f;
+        }
+        __syncthreads();
+        if (n < N) {
+            for (int k = 0; k < kc; ++k) {
+                const float w = to_f32(W[(size_t)(k0 + k) * N + n]);
+#pragma unroll
+                for (int i = 0; i < HL_TT; ++i) acc[i] = fmaf(xs[i][k], w, acc[i]);
+            }
+        }
+    }
+    if (n < N) {
+#pragma unroll
+        for (int i = 0; i < HL_TT; ++i) {
+            if (i >= nt) break;
+            float v = acc[i];
+            if (gate) {
+                const float gz = to_f32(gate[(size_t)(t0 + i) * gate_row + (size_t)h * N + n]);
+                v *= 1.0f / (1.0f + expf(-gz));
+            }
+            out[(size_t)(t0 + i) * out_row + (size_t)h * out_head + n] = from_f32<T>(v);
+        }
+    }
+    if (blockIdx.z == 0 && tl.pad_to > N) {
+        const int extra = tl.pad_to - N;
+        for (int i = tid; i < nt * extra; i += 256) {
+            const int tt = i / extra, e = i - tt * extra;
+            const T* xr = x + (size_t)(t0 + tt) * x_row + (size_t)h * x_head + K;
+            float v = 0.f;
+            if (e < tl.tail) {
+                v = to_f32(xr[e]);
+                if (e < tl.rot_dims) {
+                    const int pos = min(max(tl.positions[t0 + tt], 0), tl.max_pos - 1);
+                    const float* cs = tl.cos_sin + ((size_t)pos * (tl.rot_dims >> 1) + (e >> 1)) * 2;
+                    const float u = to_f32(xr[e & ~1]), w = to_f32(xr[e | 1]);
+                    v = (e & 1) ? fmaf(w, cs[0], u * cs[1]) : fmaf(u, cs[0], -(w * cs[1]));
+                }
+            }
+            out[(size_t)(t0 + tt) * out_row + (size_t)h * out_head + N + e] = from_f32<T>(v);
+        }
+    }
+}
+
+TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt, void* out, int out_row, int out_head,
+                            int T, int H, int K, int N, const void* gate, int gate_row, int tail, int rot_dims,
+                            int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
+                            tff_stream_t stream) {
+    TFF_REQUIRE(x && Wt && out, "head_linear: null pointer");
+    TFF_REQUIRE(T >= 0 && H > 0 && K > 0 && N > 0 && H <= 65535, "head_linear: bad sizes T=%d H=%d K=%d N=%d", T, H, K, N);
+    TFF_REQUIRE(x_head >= K + tail && x_row >= (H - 1) * x_head + K + tail,
+                "head_linear: input rows of %d with heads %d apart do not hold %d heads of %d + %d", x_row, x_head, H, K, tail);
+    const int width = pad_to > N ? pad_to : N;
+    TFF_REQUIRE(tail >= 0 && width >= N + tail && out_head >= width && out_row >= (H - 1) * out_head + width,
+                "head_linear: output rows of %d with heads %d apart do not hold %d heads of %d", out_row, out_head, H, width);
+    TFF_REQUIRE(rot_dims >= 0 && rot_dims <= tail && rot_dims % 2 == 0 && (rot_dims == 0 || (cos_sin && positions && max_pos > 0)),
+                "head_linear: %d rotated dimensions of a tail of %d need an even count, a table and positions", rot_dims, tail);
+    TFF_REQUIRE(!gate || gate_row >= H * N, "head_linear: gate rows of %d hold fewer than %d", gate_row, H * N);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const HeadLinearTail tl{tail, rot_dims, pad_to, max_pos, cos_sin, positions};
+    const dim3 grid((T + HL_TT - 1) / HL_TT, H, (N + 255) / 256);
+    if (dtype == TFF_F32)
+        head_linear_kernel<float><<<grid, 256, 0, s>>>((const float*)x, x_row, x_head, (const float*)Wt, (float*)out, out_row,
+                                                       out_head, T, K, N, (const float*)gate, gate_row, tl);
+    else if (dtype == TFF_BF16)
+        head_linear_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)Wt, (bf16_t*)out,
+                                                        out_row, out_head, T, K, N, (const bf16_t*)gate, gate_row, tl);
+    else
+        return tff_fail("head_linear: unknown dtype %d", dtype);
+    return tff_check_launch("head_linear");
+}

@@ -1,0 +1,196 @@
+// A feed-forward made of many small experts of which every token uses a few.
+//
+// tff_route_topk:   z = Wr h in float32, s = sigmoid(z); the `top` experts with the largest
+//                   s + bias are chosen (the lowest index among equals), their weights are
+//                   s / (sum of the chosen s + 1e-20): the bias moves the choice only.
+// tff_experts_gate_up: for every (token, chosen expert): g = min(Wg h, limit),
+//                   u = clamp(Wu h, -limit, limit), y = g * sigmoid(act_alpha * g) * (u + 1).
+// tff_experts_down: out[t] = sum over the token's experts, in the order they were chosen, of
+//                   weight * (Wd y), float32.
+//
+// The two expert kernels give every (token, expert) pair waves of its own that stream the
+// expert's rows once: what a step of few tokens is bound by.  Each output element is one
+// wave's dot product in a fixed order of k, so a token's result does not depend on what else
+// the step holds.  Expert weights lie [experts, out, in], row-major.
+#include "common.h"
+#include "tffinfer_kernels.h"
+
+// dot product of two rows of K elements by one wave (lanes stride through k, then a tree)
+template <typename TA, typename TB>
+__device__ __forceinline__ float wave_dot(const TA* __restrict__ a, const TB* __restrict__ b, int K, int lane) {
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) acc = fmaf(to_f32(a[k]), to_f32(b[k]), acc);
+    return wave_sum(acc);
+}
+// both rows bfloat16, K a multiple of 8 and both 16-byte aligned: eight elements a load
+__device__ __forceinline__ float wave_dot8(const bf16_t* __restrict__ a, const bf16_t* __restrict__ b, int K, int lane) {
+    float acc = 0.f;
+    for (int k = lane * 8; k < K; k += 512) {
+        union { uint4 u; bf16_t h[8]; } x, y;
+        x.u = *reinterpret_cast<const uint4*>(a + k);
+        y.u = *reinterpret_cast<const uint4*>(b + k);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = fmaf((float)x.h[j], (float)y.h[j], acc);
+    }
+    return wave_sum(acc);
+}
+template <typename T>
+__device__ __forceinline__ float row_dot(const T* a, const T* b, int K, int lane, bool vec) {
+    return wave_dot(a, b, K, lane);
+}
+template <>
+__device__ __forceinline__ float row_dot<bf16_t>(const bf16_t* a, const bf16_t* b, int K, int lane, bool vec) {
+    return vec ? wave_dot8(a, b, K, lane) : wave_dot(a, b, K, lane);
+}
+
+#define RT_MAX_E 1024
+
+template <typename T>
+__global__ __launch_bounds__(64) void route_topk_kernel(const T* __restrict__ h, int h_row, const float* __restrict__ Wr,
+                                                        const float* __restrict__ bias, int width, int E, int top,
+                                                        int32_t* __restrict__ idx, float* __restrict__ wts) {
+    __shared__ float s_all[RT_MAX_E];
+    __shared__ float c_all[RT_MAX_E];
+    __shared__ int chosen[64];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const T* hr = h + (size_t)t * h_row;
+    for (int e = 0; e < E; ++e) {
+        const float z = wave_dot(hr, Wr + (size_t)e * width, width, lane);
+        if (lane == 0) {
+            const float s = 1.0f / (1.0f + expf(-z));
+            s_all[e] = s;
+            c_all[e] = s + (bias ? bias[e] : 0.f);
+        }
+    }
+    __syncthreads();
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float c = c_all[e];
+            if (c > best) { best = c; bi = e; }      // (ascending e: the first of equals stays)
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+        }
+        __syncthreads();
+        if (lane == 0) {
+            idx[(size_t)t * top + k] = bi;
+            chosen[k] = bi;
+            c_all[bi] = -INFINITY;
+        }
+        sum += s_all[bi];
+        __syncthreads();
+    }
+    const float inv = 1.0f / (sum + 1e-20f);
+    if (lane < top) wts[(size_t)t * top + lane] = s_all[chosen[lane]] * inv;
+}
+
+TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* bias, int T, int width, int E,
+                           int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(h && Wr && idx && wts, "route_topk: null pointer");
+    TFF_REQUIRE(T >= 0 && width > 0 && h_row >= width, "route_topk: bad sizes T=%d width=%d row=%d", T, width, h_row);
+    TFF_REQUIRE(E > 0 && E <= RT_MAX_E && top > 0 && top <= E && top <= 64,
+                "route_topk: %d of %d experts (up to 64 of up to %d)", top, E, RT_MAX_E);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TFF_F32)
+        route_topk_kernel<float><<<T, 64, 0, s>>>((const float*)h, h_row, Wr, bias, width, E, top, idx, wts);
+    else if (dtype == TFF_BF16)
+        route_topk_kernel<bf16_t><<<T, 64, 0, s>>>((const bf16_t*)h, h_row, Wr, bias, width, E, top, idx, wts);
+    else
+        return tff_fail("route_topk: unknown dtype %d", dtype);
+    return tff_check_launch("route_topk");
+}
+
+#define EX_WAVES 4
+#define EX_PER_WAVE 8      // outputs a wave works through
+
+template <typename T>
+__global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
+    const T* __restrict__ h, int h_row, const T* __restrict__ Wg, const T* __restrict__ Wu,
+    const int32_t* __restrict__ idx, int top, int width, int ff, float limit, float act_alpha, T* __restrict__ y) {
+    const int pair = blockIdx.x;                  // token * top + k
+    const int t = pair / top;
+    const int e = idx[pair];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const T* hr = h + (size_t)t * h_row;
+    const T* wg = Wg + (size_t)e * ff * width;
+    const T* wu = Wu + (size_t)e * ff * width;
+    const bool vec = sizeof(T) == 2 && width % 8 == 0 && h_row % 8 == 0 && ((uintptr_t)h % 16) == 0 &&
+                     ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0;
+    const int f0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
+    for (int f = f0; f < min(ff, f0 + EX_PER_WAVE); ++f) {
+        float g = row_dot<T>(hr, wg + (size_t)f * width, width, lane, vec);
+        float u = row_dot<T>(hr, wu + (size_t)f * width, width, lane, vec);
+        if (lane == 0) {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+            const float a = g * (1.0f / (1.0f + expf(-act_alpha * g))) * (u + 1.0f);
+            y[(size_t)pair * ff + f] = from_f32<T>(a);
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
+    const T* __restrict__ y, const T* __restrict__ Wd, const int32_t* __restrict__ idx, const float* __restrict__ wts,
+    int top, int width, int ff, float* __restrict__ out) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const bool vec = sizeof(T) == 2 && ff % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)Wd % 16) == 0;
+    const int n0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
+    for (int n = n0; n < min(width, n0 + EX_PER_WAVE); ++n) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = idx[(size_t)t * top + k];
+            const float d = row_dot<T>(y + ((size_t)t * top + k) * ff, Wd + ((size_t)e * width + n) * ff, ff, lane, vec);
+            acc = fmaf(wts[(size_t)t * top + k], d, acc);
+        }
+        if (lane == 0) out[(size_t)t * width + n] = acc;
+    }
+}
+
+TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
+                                int top, int E, int width, int ff, float limit, float act_alpha, void* y, int dtype,
+                                tff_stream_t stream) {
+    TFF_REQUIRE(h && Wg && Wu && idx && y, "experts_gate_up: null pointer");
+    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width,
+                "experts_gate_up: bad sizes T=%d top=%d width=%d ff=%d", T, top, width, ff);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T * top, (ff + EX_WAVES * EX_PER_WAVE - 1) / (EX_WAVES * EX_PER_WAVE));
+    TFF_REQUIRE(grid.y <= 65535, "experts_gate_up: too many outputs");
+    if (dtype == TFF_F32)
+        experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)h, h_row, (const float*)Wg, (const float*)Wu,
+                                                                    idx, top, width, ff, limit, act_alpha, (float*)y);
+    else if (dtype == TFF_BF16)
+        experts_gate_up_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)h, h_row, (const bf16_t*)Wg,
+                                                                     (const bf16_t*)Wu, idx, top, width, ff, limit,
+                                                                     act_alpha, (bf16_t*)y);
+    else
+        return tff_fail("experts_gate_up: unknown dtype %d", dtype);
+    return tff_check_launch("experts_gate_up");
+}
+
+TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
+                             int width, int ff, float* out, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(y && Wd && idx && wts && out, "experts_down: null pointer");
+    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0, "experts_down: bad sizes T=%d top=%d width=%d ff=%d",
+                T, top, width, ff);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T, (width + EX_WAVES * EX_PER_WAVE - 1) / (EX_WAVES * EX_PER_WAVE));
+    TFF_REQUIRE(grid.y <= 65535, "experts_down: too many outputs");
+    if (dtype == TFF_F32)
+        experts_down_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)y, (const float*)Wd, idx, wts, top, width, ff, out);
+    else if (dtype == TFF_BF16)
+        experts_down_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)y, (const bf16_t*)Wd, idx, wts, top, width, ff, out);
+    else
+        return tff_fail("experts_down: unknown dtype %d", dtype);
+    return tff_check_launch("experts_down");
+}

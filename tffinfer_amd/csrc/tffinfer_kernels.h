@@ -98,12 +98,15 @@ TFF_API int tff_qk_norm_rope_kv(void* qkv, int T, int nq, int nkv, int d,
 // token_req[t] names the row of block_tables; token t sees keys at positions
 // max(0, pos-window+1) .. pos of that request (window 0: from 0).
 // Works for every head size that is a multiple of 8 up to 512.
+// sinks (float32 [nq], may be null; so for every attention entry point that takes them): a number
+// per query head whose exponential stands in the softmax's denominator beside the keys' terms,
+// with no key and no value, not scaled, counted once.
 TFF_API int tff_attention_generic(const void* q, int q_stride, void* out,
                                   const void* k_cache, const void* v_cache,
                                   const int32_t* block_tables, int bt_stride,
                                   const int32_t* token_req, const int32_t* positions,
                                   int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                  int window, float scale, int dtype, int cache_dtype,
+                                  int window, float scale, const float* sinks, int dtype, int cache_dtype,
                                   tff_stream_t stream);
 
 // bfloat16 attention on the matrix cores.  A wave works on `cols_per_wave` (16)
@@ -129,7 +132,7 @@ TFF_API int tff_attention_mfma(const void* q, int q_stride, void* out, float* pa
                                const int32_t* block_items, int num_blocks,
                                int tiles_per_entry, int cols_per_wave, int key_groups, int splits, int T_total,
                                int nq, int nkv, int d, int page_size, int num_pages, int window,
-                               float scale, tff_stream_t stream);
+                               float scale, const float* sinks, tff_stream_t stream);
 // Decoding steps (every entry brings one token), bfloat16, from the fused projection's output:
 // row r of qkv ([R, (nq + 2 nkv) d], q heads first, then k, then v) is token r.  The kernel
 // does what tff_qk_norm_rope_kv and tff_attention_mfma do one after the other, in one pass:
@@ -154,7 +157,7 @@ TFF_API int tff_attention_decode_fused(const void* qkv, int qkv_stride, void* ou
 // rows (may be null: entry i is token i for all R_total) holds (entry, token) pairs.
 TFF_API int tff_attention_split_reduce(const float* part_o, const float* part_ml, void* out,
                                        int splits, int R_total, int nq, int d, const int32_t* rows,
-                                       int num_rows, tff_stream_t stream);
+                                       int num_rows, const float* sinks, tff_stream_t stream);
 
 // tff_attention_decode_fused with every entry's keys dealt into runs by the caller, who knows
 // the entries' lengths, and the merge of the partial results, in one call.  key_runs
@@ -196,7 +199,7 @@ TFF_API int tff_attention_mfma_runs(const void* q, int q_stride, void* out, floa
                                     const int32_t* key_runs, const int32_t* run_start,
                                     const int32_t* tokens, int num_runs, int num_entries, int merge,
                                     int T, int nq, int nkv, int d, int page_size, int num_pages,
-                                    int window, float scale, tff_stream_t stream);
+                                    int window, float scale, const float* sinks, tff_stream_t stream);
 
 // tff_attention_decode_fused followed by tff_attention_split_reduce, for callers that cannot
 // allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
@@ -221,6 +224,49 @@ TFF_API int tff_attention_decode_fused_static(const void* qkv, int qkv_stride, v
                                               tff_stream_t stream);
 
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// ---- latent attention (latent_attention.hip) ----
+// Per token: c = rmsnorm(x[:rank]) * norm_w (eps inside the root), kr = x[rank : rank + rot] with
+// its first rot_dims elements rotated in pairs (2i, 2i+1) by cos_sin[position] ([max_pos,
+// rot_dims / 2, 2]); written to the token's slot (page * page_size + offset; negative: not
+// written) of a cache of ONE key head of size Dp >= rank + rot: key row [c | kr | zeros], value
+// rows (transposed page [Dp, page_size]) c in the first rank rows.
+TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, int rot, int rot_dims,
+                                const float* norm_w, float eps, const float* cos_sin, int max_pos,
+                                const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
+                                int page_size, int num_pages, int Dp, int dtype, tff_stream_t stream);
+// Products per head: out[t, h * out_head + n] = sum_k x[t, h * x_head + k] * Wt[h, k, n], Wt [H, K, N].
+// gate (may be null): the result is multiplied by sigmoid(gate[t, h * N + n]).  tail > 0: the
+// `tail` elements of the input head behind the K multiplied ones are copied behind the N results,
+// the first rot_dims of them rotated in pairs (2i, 2i+1) by the token's position; pad_to > N + tail:
+// zeros up to there.
+TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt, void* out, int out_row, int out_head,
+                            int T, int H, int K, int N, const void* gate, int gate_row, int tail, int rot_dims,
+                            int pad_to, const float* cos_sin, int max_pos, const int32_t* positions, int dtype,
+                            tff_stream_t stream);
+
+// ---- a norm after the residual sum, and the gelu (postnorm.hip) ----
+// v = alpha * resid + delta (delta may be null, or delta_planes partial sums delta_plane apart);
+// resid <- v * rsqrt(mean(v^2) + eps) * weight, in place, and out (may be null) the same rows in out_dtype.
+TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_planes, size_t delta_plane, float alpha,
+                                  const float* weight, float eps, void* out, int n, int H, int out_dtype,
+                                  tff_stream_t stream);
+// tanh_form 0: 0.5 z (1 + erf(z / sqrt 2)); 1: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dtype, tff_stream_t stream);
+
+// ---- routed experts (routed_experts.hip) ----
+// Router: s = sigmoid(Wr h) in float32 (Wr [E, width] float32); the `top` largest s + bias (bias may
+// be null) are chosen; idx [T, top], wts [T, top] = s / (sum of the chosen s + 1e-20).
+TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* bias, int T, int width, int E,
+                           int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
+// y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + 1), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
+// e = idx[t, k]; Wg, Wu [E, ff, width].
+TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
+                                int top, int E, int width, int ff, float limit, float act_alpha, void* y, int dtype,
+                                tff_stream_t stream);
+// out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff]; out float32.
+TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
+                             int width, int ff, float* out, int dtype, tff_stream_t stream);
+
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 
 // Element type conversion of n elements.

@@ -416,9 +416,10 @@ def qk_norm_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int,
 def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, block_tables: torch.Tensor, token_req: torch.Tensor,
                       positions: torch.Tensor, window: int = 0, scale: float | None = None,
-                      out: torch.Tensor | None = None) -> torch.Tensor:
+                      out: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of each token over its request's pages; q is [T, >= nq*d]
-    with the query heads at the start of each row.  Returns [T, nq*d]."""
+    with the query heads at the start of each row.  Returns [T, nq*d].
+    ``sinks`` (float32 [nq]): see :func:`paged_attention`."""
     _req(q, "attention q", ndim=2)
     T = q.shape[0]
     if q.shape[1] < nq * d:
@@ -435,13 +436,21 @@ def attention_generic(q: torch.Tensor, nq: int, nkv: int, d: int, k_cache: torch
         scale = 1.0 / math.sqrt(d)
     if out is None:
         out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
+    _check_sinks(sinks, nq)
     L = _lib.load()
     _lib.check(L.tff_attention_generic(
         q.data_ptr(), q.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
         block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(),
-        T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale),
+        T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks),
         dtype_code(q.dtype), dtype_code(k_cache.dtype), _stream()))
     return out
+
+
+def _check_sinks(sinks, nq: int) -> None:
+    if sinks is not None:
+        _req(sinks, "attention sinks", torch.float32, 1)
+        if sinks.numel() != nq:
+            raise _lib.KernelError(f"attention sinks: {sinks.numel()} numbers for {nq} query heads")
 
 
 def mfma_attention_supported(dtype: torch.dtype, d: int, page_size: int) -> bool:
@@ -596,7 +605,7 @@ def pick_splits(waves: int, max_context: int) -> int:
 def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
                    scale: float | None = None, splits: int | None = None,
                    block_bins: int | None = None, key_groups: int | None = None,
-                   block_cols: int | None = None) -> torch.Tensor:
+                   block_cols: int | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 attention of the step's tokens on the matrix cores; decode-only
     steps split each request's keys over several waves and merge them.
     ``splits``, ``block_bins`` (blocks per kv head that share the work of
@@ -622,6 +631,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     out = torch.empty(T, nq * d, dtype=q.dtype, device=q.device)
+    _check_sinks(sinks, nq)
     L = _lib.load()
     stream = _stream()
 
@@ -636,11 +646,11 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
             v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(),
             batch.start_pos.data_ptr(), _ptr(work), num_work, _ptr(block_items), num_blocks, tiles, cols,
             groups, splits, R if splits > 1 else T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window),
-            float(scale), stream))
+            float(scale), _ptr(sinks), stream))
         if splits > 1:
             _lib.check(L.tff_attention_split_reduce(
                 part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R, nq, d, _ptr(rows),
-                0 if rows is None else rows.shape[0], stream))
+                0 if rows is None else rows.shape[0], _ptr(sinks), stream))
 
     if batch.max_new_tokens == 1:
         # decoding only: a wave per request, kv head and run of keys; sizes come from the tables
@@ -655,7 +665,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
                 v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
                 runs.data_ptr(), kv.run_start.data_ptr(), batch.cu_tokens.data_ptr(), runs.shape[0], R,
                 1 if kv.runs_merge else 0, T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale),
-                stream))
+                _ptr(sinks), stream))
             return out
         if splits is None:
             splits = pick_splits(R * tiles * nkv, batch.max_context)
@@ -693,7 +703,7 @@ def attention_mfma(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window
                 q.data_ptr(), q.stride(0), out.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), k_cache.data_ptr(),
                 v_cache.data_ptr(), bt.data_ptr(), bt.stride(0), batch.cu_tokens.data_ptr(), batch.start_pos.data_ptr(),
                 runs.data_ptr(), run_start.data_ptr(), tokens.data_ptr(), runs.shape[0], len(single), 1 if merge else 0,
-                T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), stream))
+                T, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), _ptr(sinks), stream))
         else:
             work = _attention_work(batch, G, 16, q.device, "single")
             if "single_rows" not in cache:
@@ -823,7 +833,7 @@ def attention_decode_fused(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weigh
         splits, R, nq, nkv, d, k_cache.shape[2], k_cache.shape[0], int(window), float(scale), stream))
     if splits > 1:
         _lib.check(L.tff_attention_split_reduce(part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), splits, R,
-                                                nq, d, None, 0, stream))
+                                                nq, d, None, 0, None, stream))
     return out
 
 
@@ -849,15 +859,195 @@ def qkv_attention(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weig
 
 
 def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, kv, batch, window: int = 0,
-                    scale: float | None = None) -> torch.Tensor:
+                    scale: float | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of a step's tokens over the cache view ``kv`` (k_cache,
     v_cache, block_tables) with the step's ``batch``.  bfloat16 with a head
     size the matrix-core kernel takes runs there; everything else (float32,
-    other head sizes) on the general kernel."""
+    other head sizes) on the general kernel.  ``sinks`` (float32 [nq]): a
+    number per query head whose exponential is one more term of the softmax's
+    denominator, with no key and no value, not scaled."""
     if mfma_attention_supported(q.dtype, d, kv.k_cache.shape[2]):
-        return attention_mfma(q, nq, nkv, d, kv, batch, window, scale)
+        return attention_mfma(q, nq, nkv, d, kv, batch, window, scale, sinks=sinks)
     return attention_generic(q, nq, nkv, d, kv.k_cache, kv.v_cache, kv.block_tables,
-                             batch.token_req, batch.positions, window, scale)
+                             batch.token_req, batch.positions, window, scale, sinks=sinks)
+
+
+MFMA_HEAD_SIZES = tuple(range(16, 129, 16)) + (192, 256)
+
+
+def padded_head_size(d: int, dtype: torch.dtype) -> int:
+    """The head size a cache is laid out for when the attention's own is ``d``: the next size
+    the matrix-core kernels take (bfloat16; beyond their largest, and in float32, the next
+    multiple of 8, which the general kernel takes)."""
+    if dtype == torch.bfloat16:
+        for s in MFMA_HEAD_SIZES:
+            if s >= d:
+                return s
+    return -(-d // 8) * 8
+
+
+def latent_kv_store(x: torch.Tensor, rank: int, rot: int, norm_w: torch.Tensor, eps: float,
+                    cos_sin: torch.Tensor | None, positions: torch.Tensor, slot_mapping: torch.Tensor,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """Rows x [T, >= rank + rot] (rows may be strided): the RMS norm of the first ``rank`` elements
+    times ``norm_w`` and the next ``rot`` elements, rotated by ``cos_sin`` [max_pos, dims / 2, 2]
+    in pairs (2i, 2i+1), go to the tokens' slots of a cache of one key head of the padded size
+    (keys [pages, 1, page_size, Dp], values transposed)."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise _lib.KernelError("latent_kv_store x: expected a GPU matrix with unit inner stride")
+    T = x.shape[0]
+    if x.shape[1] < rank + rot:
+        raise _lib.KernelError(f"latent_kv_store: rows of {x.shape[1]} hold fewer than {rank} + {rot}")
+    _req(norm_w, "latent norm weight", torch.float32, 1)
+    if norm_w.numel() != rank:
+        raise _lib.KernelError(f"latent norm weight: {norm_w.numel()} elements for a rank of {rank}")
+    _req(k_cache, "k cache", x.dtype, 4)
+    _req(v_cache, "v cache", x.dtype, 4)
+    Dp = k_cache.shape[3]
+    _check_cache(k_cache, v_cache, 1, Dp, "latent_kv_store")
+    if Dp < rank + rot:
+        raise _lib.KernelError(f"latent_kv_store: a cache of head size {Dp} does not hold {rank} + {rot}")
+    dims, max_pos = 0, 0
+    if cos_sin is not None:
+        _req(cos_sin, "rotation table", torch.float32, 3)
+        max_pos, dims = cos_sin.shape[0], 2 * cos_sin.shape[1]
+        if cos_sin.shape[2] != 2 or dims > rot:
+            raise _lib.KernelError(f"rotation table {tuple(cos_sin.shape)} does not fit a rotated part of {rot}")
+    _req(positions, "positions", torch.int32, 1)
+    _req(slot_mapping, "slot_mapping", torch.int32, 1)
+    if positions.numel() != T or slot_mapping.numel() != T:
+        raise _lib.KernelError("latent_kv_store: positions and slot_mapping need one entry per token")
+    _lib.check(_lib.load().tff_latent_kv_store(
+        x.data_ptr(), x.stride(0) if T > 1 else x.shape[1], T, int(rank), int(rot), dims, norm_w.data_ptr(), float(eps),
+        _ptr(cos_sin), max_pos, positions.data_ptr(), slot_mapping.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        k_cache.shape[2], k_cache.shape[0], Dp, dtype_code(x.dtype), _stream()))
+
+
+def head_linear(x: torch.Tensor, x_head: int, weight_t: torch.Tensor, out_head: int | None = None,
+                gate: torch.Tensor | None = None, tail: int = 0, cos_sin: torch.Tensor | None = None,
+                positions: torch.Tensor | None = None) -> torch.Tensor:
+    """Products per head: x [T, >= H * x_head] (head h starts at h * x_head; rows may be strided),
+    ``weight_t`` [H, K, N]: out[t, h, :N] = x[t, h, :K] . weight_t[h].  Returns [T, H * out_head]
+    (``out_head`` >= N + tail, by default N + tail), zeros behind what is written.
+    ``gate`` [T, >= H * N] (rows may be strided): the products are multiplied by its sigmoid.
+    ``tail``: so many elements of the input head behind the K are copied behind the products, the
+    first ``2 * cos_sin.shape[1]`` of them rotated in pairs (2i, 2i+1) by the tokens' positions."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise _lib.KernelError("head_linear x: expected a GPU matrix with unit inner stride")
+    _req(weight_t, "head_linear weight", x.dtype, 3)
+    H, K, N = weight_t.shape
+    T = x.shape[0]
+    if x_head < K + tail or x.shape[1] < (H - 1) * x_head + K + tail:
+        raise _lib.KernelError(f"head_linear: rows of {x.shape[1]} do not hold {H} heads of {K} + {tail}, {x_head} apart")
+    width = N + tail
+    out_head = width if out_head is None else int(out_head)
+    if out_head < width:
+        raise _lib.KernelError(f"head_linear: an output head of {out_head} does not hold {N} + {tail}")
+    gate_row = 0
+    if gate is not None:
+        if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or gate.dtype != x.dtype \
+                or gate.shape[0] != T or gate.shape[1] < H * N:
+            raise _lib.KernelError("head_linear gate: expected [T, >= H * N] of the input's type on the GPU")
+        gate_row = gate.stride(0) if T > 1 else gate.shape[1]
+    dims, max_pos = 0, 0
+    if cos_sin is not None and tail > 0:
+        _req(cos_sin, "rotation table", torch.float32, 3)
+        _req(positions, "positions", torch.int32, 1)
+        max_pos, dims = cos_sin.shape[0], 2 * cos_sin.shape[1]
+        if cos_sin.shape[2] != 2 or dims > tail or positions.numel() != T:
+            raise _lib.KernelError(f"head_linear: rotation table {tuple(cos_sin.shape)} or positions do not fit")
+    out = torch.empty(T, H * out_head, dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().tff_head_linear(
+        x.data_ptr(), x.stride(0) if T > 1 else x.shape[1], int(x_head), weight_t.data_ptr(), out.data_ptr(),
+        H * out_head, out_head, T, H, K, N, _ptr(gate), gate_row, int(tail), dims, out_head if out_head > N else 0,
+        _ptr(cos_sin) if dims else None, max_pos, _ptr(positions) if dims else None, dtype_code(x.dtype), _stream()))
+    return out
+
+
+def scale_add_rmsnorm(resid: torch.Tensor, delta, weight: torch.Tensor, eps: float, alpha: float,
+                      out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """``resid <- rmsnorm(alpha * resid + delta) * weight`` in place on the float32 residual
+    stream (the norm of a block that norms after the sum); returns the same rows in
+    ``out_dtype`` (None: no copy).  ``delta`` may be None or what ``linear`` returns with
+    ``partials=True``."""
+    _req(resid, "scale_add_rmsnorm resid", torch.float32, 2)
+    n, H = resid.shape
+    _req(weight, "scale_add_rmsnorm weight", torch.float32, 1)
+    if weight.numel() != H:
+        raise _lib.KernelError(f"scale_add_rmsnorm: weight has {weight.numel()} elements, rows have {H}")
+    if isinstance(delta, PendingProduct):
+        delta = delta.run()
+    planes, plane = 1, 0
+    if delta is not None:
+        _req(delta, "scale_add_rmsnorm delta", torch.float32, 3 if delta.dim() == 3 else 2)
+        if tuple(delta.shape[-2:]) != tuple(resid.shape):
+            raise _lib.KernelError(
+                f"scale_add_rmsnorm: delta {tuple(delta.shape)} does not match resid {tuple(resid.shape)}")
+        if delta.dim() == 3:
+            planes, plane = delta.shape[0], delta.stride(0)
+    out = torch.empty(n, H, dtype=out_dtype, device=resid.device) if out_dtype is not None else None
+    _lib.check(_lib.load().tff_scale_add_rmsnorm(
+        resid.data_ptr(), _ptr(delta), planes, plane, float(alpha), weight.data_ptr(), float(eps), _ptr(out), n, H,
+        dtype_code(out_dtype) if out_dtype is not None else 0, _stream()))
+    return out
+
+
+def gelu(x: torch.Tensor, tanh_form: bool = False) -> torch.Tensor:
+    """0.5 z (1 + erf(z / sqrt 2)), or the tanh form, element by element, in float32."""
+    _req(x, "gelu input")
+    out = torch.empty_like(x)
+    _lib.check(_lib.load().tff_gelu(x.data_ptr(), out.data_ptr(), x.numel(), 1 if tanh_form else 0,
+                                    dtype_code(x.dtype), _stream()))
+    return out
+
+
+def route_topk(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int):
+    """s = sigmoid(h . router^T) in float32 (router float32 [E, width]); the ``top`` experts with
+    the largest s + bias; returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20))."""
+    _req(h, "route_topk h", ndim=2)
+    _req(router, "router", torch.float32, 2)
+    T, width = h.shape
+    E = router.shape[0]
+    if router.shape[1] != width:
+        raise _lib.KernelError(f"route_topk: router {tuple(router.shape)} for rows of {width}")
+    if bias is not None:
+        _req(bias, "router bias", torch.float32, 1)
+        if bias.numel() != E:
+            raise _lib.KernelError(f"route_topk: {bias.numel()} bias terms for {E} experts")
+    idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    _lib.check(_lib.load().tff_route_topk(h.data_ptr(), width, router.data_ptr(), _ptr(bias), T, width, E, int(top),
+                                          idx.data_ptr(), wts.data_ptr(), dtype_code(h.dtype), _stream()))
+    return idx, wts
+
+
+def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                   idx: torch.Tensor, wts: torch.Tensor, limit: float, act_alpha: float) -> torch.Tensor:
+    """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + 1) with
+    g = min(Wg h, limit), u = clamp(Wu h, -limit, limit); out = sum_k wts[:, k] Wd y.
+    ``w_gate``, ``w_up`` [E, ff, width], ``w_down`` [E, width, ff] of h's type; float32 [T, width]."""
+    _req(h, "routed_experts h", ndim=2)
+    T, width = h.shape
+    for w, nm in ((w_gate, "gate"), (w_up, "up"), (w_down, "down")):
+        _req(w, f"experts {nm}", h.dtype, 3)
+    E, ff, _ = w_gate.shape
+    if tuple(w_gate.shape) != (E, ff, width) or tuple(w_up.shape) != (E, ff, width) \
+            or tuple(w_down.shape) != (E, width, ff):
+        raise _lib.KernelError(f"routed_experts: weights {tuple(w_gate.shape)}, {tuple(w_up.shape)}, "
+                               f"{tuple(w_down.shape)} for rows of {width}")
+    _req(idx, "experts idx", torch.int32, 2)
+    _req(wts, "experts weights", torch.float32, 2)
+    top = idx.shape[1]
+    if tuple(idx.shape) != (T, top) or tuple(wts.shape) != (T, top):
+        raise _lib.KernelError("routed_experts: idx and weights must be [T, top]")
+    L = _lib.load()
+    y = torch.empty(T * top, ff, dtype=h.dtype, device=h.device)
+    _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), idx.data_ptr(), T, top, E,
+                                     width, ff, float(limit), float(act_alpha), y.data_ptr(), dtype_code(h.dtype), _stream()))
+    out = torch.empty(T, width, dtype=torch.float32, device=h.device)
+    _lib.check(L.tff_experts_down(y.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(), T, top, E, width, ff,
+                                  out.data_ptr(), dtype_code(h.dtype), _stream()))
+    return out
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -992,6 +1182,12 @@ OP_TABLE = {
     "attention_decode_fused": attention_decode_fused,
     "qkv_attention": qkv_attention,
     "swiglu": swiglu,
+    "latent_kv_store": latent_kv_store,
+    "head_linear": head_linear,
+    "scale_add_rmsnorm": scale_add_rmsnorm,
+    "gelu": gelu,
+    "route_topk": route_topk,
+    "routed_experts": routed_experts,
     "cast": cast,
     "argmax": argmax,
     "repetition_penalty": repetition_penalty,

@@ -16,7 +16,7 @@ from ..config.base import ModelConfig
 from ..parts.base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, WeightSpec
 from ..parts.embedding import Embedding, OutputHead
 from ..weights.loader import check_weights, normalize_stored
-from ..weights.random_init import random_tensor
+from ..weights.random_init import FLOAT32_INITS, random_tensor
 
 
 @dataclass
@@ -30,6 +30,15 @@ class TensorNames:
     children: dict = field(default_factory=dict)
     #: tensors a file may hold that the model has no use for
     ignorable: tuple = ()
+    #: True: a part's tensor called "weight" carries the part's own name in the file
+    #: ("final.norm", not "final.norm.weight"); a part's other tensors follow the part's name
+    bare_weights: bool = False
+
+    def tensor(self, prefix: str, local: str) -> str:
+        """The file's name of the tensor ``local`` of the part named ``prefix``."""
+        if self.bare_weights and local == "weight":
+            return prefix
+        return f"{prefix}.{local}"
 
 
 def _leaves(prefix: str, part: Part, rename: dict):
@@ -55,6 +64,12 @@ class DecoderModel:
             block = BLOCKS.build(spec.block, mixer=mixer, feed_forward=ffn,
                                  make_norm=lambda s=norm_spec: NORMS.build(s))
             self.blocks.append(block)
+        # the number each layer with tensors has in the file's names (layers that borrow another
+        # layer's tensors are calls of that layer in the run order and have no number here)
+        numbers = getattr(config, "layer_numbers", None)
+        self.layer_numbers = list(numbers()) if callable(numbers) else list(range(len(self.blocks)))
+        if len(self.layer_numbers) != len(self.blocks):
+            raise ValueError("the configuration numbers another count of layers than it specifies")
         self.schedule = list(config.layer_schedule())
         for call in self.schedule:
             if not 0 <= call.layer < len(self.blocks):
@@ -65,7 +80,7 @@ class DecoderModel:
     # ---- weights ---------------------------------------------------------
     def _weighted_parts(self):
         yield self.names.embedding, self.embedding
-        for i, block in enumerate(self.blocks):
+        for i, block in zip(self.layer_numbers, self.blocks):
             yield from _leaves(self.names.layer.format(i=i), block, self.names.children)
         yield self.names.final_norm, self.final_norm
         yield self.names.head, self.head
@@ -74,7 +89,7 @@ class DecoderModel:
         out = {}
         for prefix, part in self._weighted_parts():
             for local, spec in part.weight_specs().items():
-                out[f"{prefix}.{local}"] = spec
+                out[self.names.tensor(prefix, local)] = spec
         return out
 
     def load_tensors(self, found: dict[str, torch.Tensor], dtype: torch.dtype, device,
@@ -83,7 +98,7 @@ class DecoderModel:
         that is wrong) and hands every part its tensors."""
         ignorable = set(self.names.ignorable)
         if self.config.tie_word_embeddings:
-            head = f"{self.names.head}.weight"
+            head = self.names.tensor(self.names.head, "weight")
             ignorable.add(head)
             if head in found:
                 from .. import log
@@ -94,7 +109,8 @@ class DecoderModel:
         for prefix, part in self._weighted_parts():
             specs = part.weight_specs()
             if specs:
-                part.load_weights({local: normalize_stored(found[f"{prefix}.{local}"]) for local in specs},
+                part.load_weights({local: normalize_stored(found[self.names.tensor(prefix, local)])
+                                   for local in specs if self.names.tensor(prefix, local) in found},
                                   dtype, self.device)
 
     def init_random(self, seed: int, dtype: torch.dtype, device, on_device: bool = False) -> None:
@@ -107,8 +123,10 @@ class DecoderModel:
             if specs:
                 ws = {}
                 for local, spec in specs.items():
-                    t = random_tensor(spec, seed, f"{prefix}.{local}", device=gen_dev)
-                    ws[local] = t if spec.init == "norm" else t.to(torch.bfloat16)
+                    if spec.optional:
+                        continue
+                    t = random_tensor(spec, seed, self.names.tensor(prefix, local), device=gen_dev)
+                    ws[local] = t if spec.init in FLOAT32_INITS else t.to(torch.bfloat16)
                 part.load_weights(ws, dtype, self.device)
 
     def graph_safe(self) -> bool:

@@ -50,11 +50,20 @@ def registered_architectures() -> list[str]:
     return sorted(_ARCHITECTURES)
 
 
-def config_from_dict(d: dict) -> ModelConfig:
+def architecture_name(d: dict) -> str:
+    """The name a config.json files its model under: the first of 'architectures', or the
+    string 'architecture' of files that name one only."""
     archs = d.get("architectures")
-    if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json: required key 'architectures' (a list of names) is missing")
-    return get_architecture(archs[0]).config_cls.from_dict(d)
+    if isinstance(archs, list) and archs and isinstance(archs[0], str):
+        return archs[0]
+    if isinstance(d.get("architecture"), str):
+        return d["architecture"]
+    raise ConfigError("config.json: required key 'architectures' (a list of names) or 'architecture' (a name) "
+                      "is missing")
+
+
+def config_from_dict(d: dict) -> ModelConfig:
+    return get_architecture(architecture_name(d)).config_cls.from_dict(d)
 
 
 def load_config(model_dir: str) -> ModelConfig:

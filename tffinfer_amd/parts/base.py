@@ -28,9 +28,12 @@ from ..config.base import ConfigError, PartSpec
 @dataclass(frozen=True)
 class WeightSpec:
     """Shape of a weight tensor and the law random weights follow:
-    ``matrix`` N(0, 0.02), ``norm`` 1 + N(0, 0.1), ``embedding`` N(0, 0.02)."""
+    ``matrix`` N(0, 0.02), ``norm`` 1 + N(0, 0.1), ``norm_offset`` N(0, 0.1) (a norm weight
+    stored around zero), ``vector`` N(0, 0.5), ``embedding`` N(0, 0.02).
+    ``optional``: a file may leave the tensor out, and the part then does without it."""
     shape: tuple
     init: str = "matrix"
+    optional: bool = False
 
 
 @dataclass(frozen=True)

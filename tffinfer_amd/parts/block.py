@@ -39,3 +39,50 @@ class PreNormBlock(Block):
         a = self.mixer.forward(ctx, h)
         z = self._norm(self.norm2, self.feed_forward, ctx, resid, a)
         return self.feed_forward.forward(ctx, z)
+
+
+@register_block("postnorm")
+class PostNormBlock(Block):
+    """x <- norm1(alpha x + mixer(x));  x <- norm2(alpha x + ffn(x)): the norms stand after the
+    sums, on the stream itself, and the sublayers read the stream as it is.  The float32
+    residual stream therefore holds normed rows; each norm also leaves them in the activation
+    type for the products that read them next, and the block hands that copy to the block
+    after it through the step's batch.  A layer without a feed-forward has no second sum; its
+    second norm runs only if the file holds a weight for it."""
+
+    graph_safe = True
+
+    def __init__(self, mixer, feed_forward, make_norm, alpha: float = 1.0):
+        self.alpha = float(alpha)
+        self.norm1 = make_norm()
+        self.mixer = mixer
+        self.norm2 = make_norm()
+        self.feed_forward = feed_forward
+        self.has_ffn = not getattr(feed_forward, "is_none", False)
+        if not self.has_ffn:
+            self.norm2.optional = True
+
+    def children(self):
+        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
+                "feed_forward": self.feed_forward}
+
+    def _rows(self, ctx, resid):
+        """The stream in the activation type: what the block before left, or a cast."""
+        if ctx.act_dtype == resid.dtype:
+            return resid
+        left = getattr(ctx.batch, "_normed_rows", None)
+        if left is not None and left[0] is resid and left[1] == ctx.call_index - 1:
+            return left[2]
+        return ctx.ops.cast(resid, ctx.act_dtype)
+
+    def forward(self, ctx, resid, pending):
+        if pending is not None:
+            resid += ctx.ops.as_tensor(pending)
+        h = self._rows(ctx, resid)
+        h = self.norm1.forward_post(ctx, resid, self.mixer.forward(ctx, h), self.alpha)
+        if self.has_ffn:
+            h = self.norm2.forward_post(ctx, resid, self.feed_forward.forward(ctx, h), self.alpha)
+        elif self.norm2.weight is not None:
+            h = self.norm2.forward_post(ctx, resid, None, self.alpha)
+        ctx.batch._normed_rows = (resid, ctx.call_index, h)
+        return None

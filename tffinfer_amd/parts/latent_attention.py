@@ -1,0 +1,125 @@
+"""Attention whose keys and values are kept as one low-rank latent vector per token."""
+from __future__ import annotations
+
+import torch
+
+from ..config.base import ConfigError, PartSpec
+from .base import (POSITION_ENCODINGS, KVCacheSpec, Mixer, PositionEncoding, WeightSpec,
+                   register_mixer, to_device)
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    """Per token t with input h:
+
+        q_h   = (Wq h)[head h] = [q_h^n (head_dim) | q_h^r (rot_dim)]
+        [a|b] = Wdkv h,  c = rmsnorm(a) * w_c  (kv_rank),  kr = b (rot_dim; shared by all heads)
+        k_h^n = Wuk_h c,  v_h = Wuv_h c
+        s_h(i, j) = (q_h^n(i) . k_h^n(j) + R_i q_h^r(i) . R_j kr(j)) * scale,  0 <= i - j < window
+        p_h(i, .) = softmax over the visible j and one sink term e^(sink_h) in the denominator
+        out = Wo [ (sum_j p_h(i, j) v_h(j)) * sigmoid(Wg h)[head h] ]_h
+
+    R_p rotates pairs (2i, 2i+1) by the position's angles.  Only c and R kr are cached.  The
+    up-projections are taken to the query's side (q_h^n . Wuk_h c = (Wuk_h^T q_h^n) . c, and
+    sum_j p v_h(j) = Wuv_h sum_j p c(j)), so the attention proper is attention with one key
+    head of size kv_rank + rot_dim whose values are the first kv_rank elements of its keys; it
+    runs on the paged attention kernels, padded to a head size they take.  Wq, Wdkv and Wg are
+    one product.
+    """
+
+    graph_safe = True
+    input_goes_to_linear = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int,
+                 kv_rank: int, scale: float, position=None, window: int = 0,
+                 latent_norm_eps: float = 1e-6, sink: bool = True, output_gate: bool = True):
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.head_dim = int(head_dim)
+        self.rot_dim = int(rot_dim)
+        self.value_dim = int(value_dim)
+        self.kv_rank = int(kv_rank)
+        self.scale = float(scale)
+        self.window = int(window or 0)
+        self.latent_norm_eps = float(latent_norm_eps)
+        self.has_sink = bool(sink)
+        self.has_gate = bool(output_gate)
+        for k in ("hidden_size", "num_heads", "head_dim", "value_dim", "kv_rank"):
+            if getattr(self, k) <= 0:
+                raise ConfigError(f"latent attention: '{k}' must be positive, found {getattr(self, k)}")
+        if self.rot_dim < 0:
+            raise ConfigError(f"latent attention: 'rot_dim' must not be negative, found {self.rot_dim}")
+        if isinstance(position, PartSpec):
+            position = POSITION_ENCODINGS.build(position)
+        if position is not None and not isinstance(position, PositionEncoding):
+            raise ConfigError("latent attention: 'position' must be a position encoding or its spec")
+        if position is not None and position.rotary_dim:
+            if position.pairing != "interleaved":
+                raise ConfigError("latent attention: the rotated part is rotated in pairs (2i, 2i+1) only")
+            if position.rotary_dim > self.rot_dim:
+                raise ConfigError(f"latent attention: {position.rotary_dim} rotated dimensions of a part of {self.rot_dim}")
+        self.position = position
+        self._dtype = torch.bfloat16
+        self.w_in = self.w_uk_t = self.w_uv_t = self.w_o = self.latent_norm = self.sink = None
+
+    # ---- sizes -----------------------------------------------------------
+    @property
+    def key_dim(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    def padded_key_dim(self) -> int:
+        from ..kernels.ops import padded_head_size
+        return padded_head_size(self.key_dim, self._dtype)
+
+    def cache_spec(self):
+        return KVCacheSpec(1, self.padded_key_dim(), self.window)
+
+    def flops_per_query_key_pair(self):
+        return 4 * self.num_heads * self.padded_key_dim()
+
+    def weight_specs(self):
+        W, H = self.hidden_size, self.num_heads
+        specs = {
+            "q": WeightSpec((H * (self.head_dim + self.rot_dim), W)),
+            "dkv": WeightSpec((self.key_dim, W)),
+            "dkv.norm": WeightSpec((self.kv_rank,), "norm"),
+            "uk": WeightSpec((H * self.head_dim, self.kv_rank)),
+            "uv": WeightSpec((H * self.value_dim, self.kv_rank)),
+            "o": WeightSpec((W, H * self.value_dim)),
+        }
+        if self.has_sink:
+            specs["sink"] = WeightSpec((H,), "vector")
+        if self.has_gate:
+            specs["g"] = WeightSpec((H * self.value_dim, W))
+        return specs
+
+    def load_weights(self, weights, dtype, device):
+        H = self.num_heads
+        self._dtype = dtype
+        stacked = [weights["q"], weights["dkv"]] + ([weights["g"]] if self.has_gate else [])
+        self.w_in = to_device(torch.cat([w.to(stacked[0].dtype) for w in stacked], 0), dtype, device)
+        self.w_o = to_device(weights["o"], dtype, device)
+        # [H, head_dim, rank]: k_h^n = Wuk_h c, so (Wuk_h^T q)[r] = sum_d q[d] Wuk[h, d, r]
+        self.w_uk_t = weights["uk"].to(dtype).view(H, self.head_dim, self.kv_rank).contiguous().to(device)
+        # [H, rank, value_dim]: v_h[e] = sum_r Wuv[h, e, r] c[r]
+        self.w_uv_t = weights["uv"].to(dtype).view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous().to(device)
+        self.latent_norm = weights["dkv.norm"].to(torch.float32).contiguous().to(device)
+        self.sink = weights["sink"].to(torch.float32).contiguous().to(device) if self.has_sink else None
+
+    def forward(self, ctx, x):
+        ops, kv, b = ctx.ops, ctx.kv, ctx.batch
+        H, rank, rot = self.num_heads, self.kv_rank, self.rot_dim
+        nq = H * (self.head_dim + rot)
+        Dp = kv.k_cache.shape[3]
+        proj = ops.linear(x, self.w_in)
+        table = None
+        if self.position is not None and self.position.rotary_dim:
+            table = self.position.cached_table(ctx.max_positions, proj.device)
+        ops.latent_kv_store(proj[:, nq:nq + rank + rot], rank, rot, self.latent_norm, self.latent_norm_eps, table,
+                            b.positions, kv.slot_mapping, kv.k_cache, kv.v_cache)
+        q = ops.head_linear(proj[:, :nq], self.head_dim + rot, self.w_uk_t, out_head=Dp, tail=rot, cos_sin=table,
+                            positions=b.positions)
+        o = ops.paged_attention(q, H, 1, Dp, kv, b, self.window, self.scale, sinks=self.sink)
+        gate = proj[:, nq + rank + rot:] if self.has_gate else None
+        o = ops.head_linear(o, Dp, self.w_uv_t, gate=gate)
+        return ops.linear(o, self.w_o, out_dtype=torch.float32, partials=True)

@@ -50,3 +50,108 @@ class SwiGLU(FeedForward):
         gu = ctx.ops.linear(x, self.w_gate_up)
         m = gu if getattr(self.w_gate_up, "glu_out", 0) else ctx.ops.swiglu(gu)
         return ctx.ops.linear(m, self.w_down, out_dtype=torch.float32, partials=True)
+
+
+@register_feed_forward("none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: the block leaves the sublayer out."""
+
+    graph_safe = True
+    is_none = True
+
+    def __init__(self, hidden_size: int = 0):
+        self.hidden_size = int(hidden_size)
+
+    def forward(self, ctx, x):
+        return None
+
+
+@register_feed_forward("gelu_mlp")
+class GeluMLP(FeedForward):
+    """f = Wdown gelu(Wup z), no gate and no biases; the gelu is the exact one,
+    0.5 z (1 + erf(z / sqrt 2)), or with ``tanh_form`` its tanh approximation."""
+
+    graph_safe = True
+    input_goes_to_linear = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, tanh_form: bool = False):
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.tanh_form = bool(tanh_form)
+        self.w_up = self.w_down = None
+
+    def weight_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        return {"up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
+
+    def load_weights(self, weights, dtype, device):
+        self.w_up = to_device(weights["up"], dtype, device)
+        self.w_down = to_device(weights["down"], dtype, device)
+
+    def forward(self, ctx, x):
+        a = ctx.ops.gelu(ctx.ops.linear(x, self.w_up), self.tanh_form)
+        return ctx.ops.linear(a, self.w_down, out_dtype=torch.float32, partials=True)
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(FeedForward):
+    """``num_experts`` small gated feed-forwards of which every token uses ``top``.
+
+        s = sigmoid(Wr z)                      (float32)
+        chosen: the ``top`` largest s + b      (b: a correction that moves the choice only)
+        w_e = s_e / (sum of the chosen s + 1e-20)
+        expert e: g = min(Wg z, limit), u = clamp(Wu z, -limit, limit),
+                  y = g * sigmoid(act_alpha * g) * (u + 1),  f_e = Wd y
+        f = sum over the chosen e of w_e f_e
+
+    The experts' matrices lie stacked, [experts, out, in], so that a kernel finds an expert's
+    rows by its number."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
+                 limit: float, act_alpha: float = 1.702, correction: bool = True):
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.num_experts = int(num_experts)
+        self.top = int(top)
+        self.limit = float(limit)
+        self.act_alpha = float(act_alpha)
+        self.has_correction = bool(correction)
+        if not 0 < self.top <= self.num_experts:
+            from ..config.base import ConfigError
+            raise ConfigError(f"routed experts: top={self.top} of {self.num_experts} experts")
+        self.w_gate = self.w_up = self.w_down = self.router = self.correction = None
+
+    def weight_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        specs = {"router": WeightSpec((self.num_experts, H))}
+        if self.has_correction:
+            specs["correction"] = WeightSpec((self.num_experts,), "vector")
+        for e in range(self.num_experts):
+            specs[f"e{e}.gate"] = WeightSpec((I, H))
+            specs[f"e{e}.up"] = WeightSpec((I, H))
+            specs[f"e{e}.down"] = WeightSpec((H, I))
+        return specs
+
+    def active_matrix_elements(self) -> int:
+        """Matrix elements a token multiplies with: the router and its ``top`` experts."""
+        H, I = self.hidden_size, self.intermediate_size
+        return self.num_experts * H + self.top * 3 * H * I
+
+    def load_weights(self, weights, dtype, device):
+        E = self.num_experts
+
+        def stack(which):
+            return torch.stack([weights[f"e{e}.{which}"].to(dtype) for e in range(E)], 0).contiguous().to(device)
+
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        self.router = weights["router"].to(torch.float32).contiguous().to(device)
+        self.correction = (weights["correction"].to(torch.float32).contiguous().to(device)
+                           if self.has_correction else None)
+
+    def forward(self, ctx, x):
+        ops = ctx.ops
+        x = ops.as_tensor(x)
+        idx, wts = ops.route_topk(x, self.router, self.correction, self.top)
+        return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha)

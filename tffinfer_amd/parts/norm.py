@@ -11,21 +11,42 @@ class RMSNorm(Norm):
     """y = v * rsqrt(mean(v^2) + eps) * w over rows of ``size`` elements, where
     v is the residual stream plus the term still pending; sum, mean, rsqrt and
     products in float32.  Reference: src/kernel/cuda/norm.cu:31-48 (the weight
-    product fused as in src/core/runtime/GraphOptimizer.cpp:197-229)."""
+    product fused as in src/core/runtime/GraphOptimizer.cpp:197-229).
+
+    ``weight_offset``: the stored weight lies around zero and the factor is
+    ``weight_offset + w`` (formed once, in float32, at load).  ``optional``: a
+    file may leave the weight out; the norm then has none and its block skips it."""
 
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, weight_offset: float = 0.0, optional: bool = False):
         self.size = int(size)
         self.eps = float(eps)
+        self.weight_offset = float(weight_offset)
+        self.optional = bool(optional)
         self.weight = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.size,), "norm")}
+        return {"weight": WeightSpec((self.size,), "norm_offset" if self.weight_offset else "norm",
+                                     optional=self.optional)}
 
     def load_weights(self, weights, dtype, device):
+        if "weight" not in weights:
+            self.weight = None
+            return
         # norm weights stay in float32 whatever the activation type is
-        self.weight = weights["weight"].to(torch.float32).contiguous().to(device)
+        w = weights["weight"].to(torch.float32)
+        if self.weight_offset:
+            w = w + self.weight_offset
+        self.weight = w.contiguous().to(device)
+
+    def forward_post(self, ctx, resid, delta, alpha: float):
+        """The norm of a block that norms after the sum: ``resid <- norm(alpha * resid + delta)``
+        in place; returns the rows in the activation type (the stream itself where that is
+        float32)."""
+        out = ctx.ops.scale_add_rmsnorm(resid, delta, self.weight, self.eps, alpha,
+                                        None if ctx.act_dtype == torch.float32 else ctx.act_dtype)
+        return resid if out is None else out
 
     #: ``forward`` takes ``for_linear``: its result may then be rows that lack the norm's factor,
     #: which only ``ops.linear`` understands

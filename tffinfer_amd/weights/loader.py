@@ -33,7 +33,7 @@ _FLOATS = (torch.float32, torch.bfloat16, torch.float16)
 def check_weights(expected: dict[str, WeightSpec], found: dict[str, torch.Tensor],
                   ignorable: set[str] = frozenset(), where: str = "") -> None:
     """Raises one WeightError naming everything that is wrong."""
-    missing = [n for n in expected if n not in found]
+    missing = [n for n in expected if n not in found and not expected[n].optional]
     unexpected = [n for n in found if n not in expected and n not in ignorable]
     wrong_shape = [(n, expected[n].shape, tuple(found[n].shape)) for n in expected
                    if n in found and tuple(found[n].shape) != tuple(expected[n].shape)]

@@ -12,6 +12,9 @@ from .safetensors_io import save_file
 
 MATRIX_STD = 0.02
 NORM_STD = 0.1
+VECTOR_STD = 0.5
+#: laws whose tensors are kept in float32 whatever the matrices are stored in
+FLOAT32_INITS = ("norm", "norm_offset", "vector")
 
 
 def tensor_seed(seed: int, name: str) -> int:
@@ -22,12 +25,17 @@ def tensor_seed(seed: int, name: str) -> int:
 
 def random_tensor(spec: WeightSpec, seed: int, name: str, device="cpu") -> torch.Tensor:
     """float32 values: matrices and embeddings N(0, 0.02), norm weights
-    1 + N(0, 0.1)."""
+    1 + N(0, 0.1) (``norm_offset``: stored around zero, N(0, 0.1)), small vectors that
+    enter scores or logits (``vector``) N(0, 0.5)."""
     g = torch.Generator(device=device)
     g.manual_seed(tensor_seed(seed, name))
     x = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device)
     if spec.init == "norm":
         return 1.0 + NORM_STD * x
+    if spec.init == "norm_offset":
+        return NORM_STD * x
+    if spec.init == "vector":
+        return VECTOR_STD * x
     return MATRIX_STD * x
 
 
@@ -42,8 +50,10 @@ def write_random_model(model_dir: str, config, seed: int, dtype: str = "bfloat16
     expected = build_model_skeleton(config).expected_tensors()
     tensors = {}
     for name, spec in expected.items():
+        if spec.optional:
+            continue        # (a tensor a file may leave out is left out)
         t = random_tensor(spec, seed, name)
-        tensors[name] = t if spec.init == "norm" else t.to(store)
+        tensors[name] = t if spec.init in FLOAT32_INITS else t.to(store)
     os.makedirs(model_dir, exist_ok=True)
     d = config.to_dict()
     d["torch_dtype"] = dtype
