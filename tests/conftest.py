@@ -21,6 +21,14 @@ def model_dirs(tmp_path_factory):
     return {name: make_model_dir(str(base / name), cfg, seed) for name, (cfg, seed) in TINY_CONFIGS.items()}
 
 
+@pytest.fixture(scope="session")
+def disunex_dirs(tmp_path_factory):
+    """Model folders of the tiny Disunex configurations (sharpened weights), once per session."""
+    from disunex_models import DISUNEX_CONFIGS, make_disunex_dir
+    base = tmp_path_factory.mktemp("disunex")
+    return {name: make_disunex_dir(str(base / name), cfg, seed) for name, (cfg, seed) in DISUNEX_CONFIGS.items()}
+
+
 @pytest.fixture(autouse=True)
 def _seeded():
     """Every test draws the same random inputs in every run."""

@@ -139,7 +139,8 @@ def run_steps_subprocess(model_dir, dtype, steps, out_dir, max_tokens, extra_arg
         if p.poll() is None:
             p.kill()
     with open(os.path.join(model_dir, "config.json")) as f:
-        V = json.load(f)["vocab_size"]
+        cfg = json.load(f)
+        V = cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"]
     out = {}
     for s in steps:
         path = os.path.join(out_dir, f"{s['step']}.f32")

@@ -95,7 +95,7 @@ class DisunexConfig(ModelConfig):
 
     architecture = ARCHITECTURE
     tie_word_embeddings = True      # the logits are products with the embedding table
-    caller_options: dict = None
+    caller_options = {}
 
     @classmethod
     def from_dict(cls, d: dict) -> "DisunexConfig":

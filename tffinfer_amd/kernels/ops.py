@@ -73,10 +73,13 @@ class PackedWeight:
     """A bfloat16 matrix [N, K] in the fragment order of the matrix-core
     products: tiles of 16 rows by 32 k stored as the 1 KB operand a wave loads,
     rows and k padded with zeros to multiples of 16 and 32."""
-    __slots__ = ("data", "N", "K", "glu_out")
+    __slots__ = ("data", "N", "K", "glu_out", "k_in")
 
-    def __init__(self, data: torch.Tensor, N: int, K: int, glu_out: int = 0):
+    def __init__(self, data: torch.Tensor, N: int, K: int, glu_out: int = 0, k_in: int | None = None):
         self.data, self.N, self.K = data, int(N), int(K)
+        #: the inner size of the matrix it was packed from, where that was no multiple of 8 (K is
+        #: the next one, the columns between are zeros; ``linear`` widens its rows to match)
+        self.k_in = int(k_in) if k_in is not None else int(K)
         #: > 0: the 16-row groups alternate between a gate and an up projection and the
         #: product yields silu(gate) * up with this many columns
         self.glu_out = int(glu_out)
@@ -110,14 +113,16 @@ class PackedWeight:
 def pack_weight(w: torch.Tensor) -> PackedWeight:
     """Row-major bfloat16 [N, K] on the GPU -> fragment order."""
     _req(w, "pack_weight", torch.bfloat16, 2)
+    N, k_in = w.shape
+    if k_in % 8:
+        # (the products take inner sizes in units of 8: zero columns change no sum)
+        w = torch.nn.functional.pad(w, (0, 8 - k_in % 8)).contiguous()
     N, K = w.shape
-    if K % 8:
-        raise _lib.KernelError(f"pack_weight: inner size {K} must be a multiple of 8")
     NB, KB = -(-N // 16), -(-K // 32)
     out = torch.empty(NB * KB * 512, dtype=torch.bfloat16, device=w.device)
     L = _lib.load()
     _lib.check(L.tff_pack_weight(w.data_ptr(), out.data_ptr(), N, K, _stream()))
-    return PackedWeight(out, N, K)
+    return PackedWeight(out, N, K, k_in=k_in)
 
 
 def pack_gate_up(gate: torch.Tensor, up: torch.Tensor) -> PackedWeight:
@@ -151,6 +156,15 @@ def embed(table, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
     _req(ids, "embed ids", torch.int32, 1)
     V, H = table.shape
     T = ids.numel()
+    if packed and table.k_in != H:
+        # (a table whose rows were widened to a multiple of 8: the rows come out as wide, and are cut)
+        wide = torch.empty(T, H, dtype=torch.float32, device=table.device)
+        _lib.check(_lib.load().tff_embed_packed(table.data_ptr(), ids.data_ptr(), wide.data_ptr(), T, H, V, _stream()))
+        cut = wide[:, :table.k_in].contiguous()
+        if out is not None:
+            out.copy_(cut)
+            return out
+        return cut
     if out is None:
         out = torch.empty(T, H, dtype=torch.float32, device=table.device)
     else:
@@ -329,6 +343,9 @@ def linear(x: torch.Tensor, weight, out_dtype: torch.dtype | None = None,
             raise _lib.KernelError("linear: a bfloat16 weight must be a PackedWeight (pack_weight)")
     M, K = x.shape
     N, K2 = weight.shape
+    if packed and K != K2 and K == weight.k_in:
+        x = torch.nn.functional.pad(x, (0, K2 - K))      # a weight whose inner size was rounded up to 8
+        K = K2
     if K != K2:
         raise _lib.KernelError(f"linear: x has inner size {K}, weight [out, in] = {tuple(weight.shape)}")
     lda = x.stride(0) if M > 1 else K
