@@ -509,13 +509,17 @@ def test_linear_identity_and_layout():
     assert torch.equal(out[:, 0], x[:, 3]) and torch.equal(out[:, 1], 2 * x[:, 7])
 
 
-def test_linear_refuses_bad_inner_size():
+def test_linear_widens_an_inner_size_that_is_no_multiple_of_8_and_refuses_a_plain_bfloat16_weight():
     from tffinfer_amd.kernels.lib import KernelError
     ops = _ops()
-    x = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
-    w = torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(KernelError, match="multiple of 8"):
-        ops.pack_weight(w)
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(4, 12, generator=g).to(torch.bfloat16)
+    w = torch.randn(9, 12, generator=g).to(torch.bfloat16)
+    pw = ops.pack_weight(w.to(DEV))          # zero columns up to 16: no sum changes
+    assert (pw.K, pw.k_in, pw.N) == (16, 12, 9)
+    _close(ops.linear(x.to(DEV), pw, out_dtype=torch.float32), x.double() @ w.double().T, 1e-5, "widened product")
+    with pytest.raises(KernelError, match="inner size"):
+        ops.linear(torch.zeros(4, 13, dtype=torch.bfloat16, device=DEV), pw)
     with pytest.raises(KernelError, match="PackedWeight"):
         ops.linear(torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV),
                    torch.zeros(8, 16, dtype=torch.bfloat16, device=DEV))
