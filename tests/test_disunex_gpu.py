@@ -82,11 +82,12 @@ def test_router_choice_goes_by_the_corrected_scores_and_weights_by_the_plain_one
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("E,top,width,ff,limit", [(5, 2, 64, 40, 0.7), (3, 1, 100, 24, 1.5), (6, 3, 72, 17, 0.5)])
-def test_experts(dtype, E, top, width, ff, limit):
+@pytest.mark.parametrize("T", [19, 150])
+@pytest.mark.parametrize("E,top,width,ff,limit", [(5, 2, 64, 40, 0.7), (3, 1, 100, 24, 1.5), (6, 3, 72, 17, 0.5),
+                                                  (40, 4, 264, 136, 0.8)])
+def test_experts(dtype, E, top, width, ff, limit, T):
     ops = _ops()
     g = torch.Generator().manual_seed(E + ff)
-    T = 19
     h = torch.randn(T, width, generator=g).to(dtype)
     wg = (torch.randn(E, ff, width, generator=g) * 0.2).to(dtype)       # large enough that both clamps bite
     wu = (torch.randn(E, ff, width, generator=g) * 0.2).to(dtype)
@@ -101,8 +102,18 @@ def test_experts(dtype, E, top, width, ff, limit):
             ref[t] += wts[t, k].double() * plain.expert(h[t].double(), wg[e].double(), wu[e].double(), wd[e].double(), limit)
             clamped += int(((h[t].double() @ wu[e].double().T).abs() > limit).sum())
     assert clamped > 0
-    out = ops.routed_experts(h.to(DEV), wg.to(DEV), wu.to(DEV), wd.to(DEV), idx.to(DEV), wts.to(DEV), limit, 1.702)
+    args = (h.to(DEV), wg.to(DEV), wu.to(DEV), wd.to(DEV), idx.to(DEV), wts.to(DEV), limit, 1.702)
+    out = ops.as_tensor(ops.routed_experts(*args))      # (150 tokens in bfloat16: dealt to the experts in tiles)
     assert _err(out, ref) < (2e-6 if dtype == torch.float32 else 1.5e-2)
+    if dtype == torch.bfloat16:
+        # a pair's row does not depend on how the pairs were dealt: the two paths agree to rounding,
+        # and a token alone gives what it gives among the others
+        few = ops.as_tensor(ops.routed_experts(*args, by_tiles=False))
+        tiles = ops.as_tensor(ops.routed_experts(*args, by_tiles=True)) if ff % 8 == 0 and width % 8 == 0 else few
+        assert _err(tiles, few) < 1e-2
+        one = [a[7:8].contiguous() if isinstance(a, torch.Tensor) and a.shape[0] == T else a for a in args]
+        alone = ops.as_tensor(ops.routed_experts(*one, by_tiles=ff % 8 == 0 and width % 8 == 0))
+        assert torch.equal(alone[0], tiles[7])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -141,22 +152,23 @@ def test_latent_vector_and_rotated_key_go_to_their_slots(dtype, rank, rot, dims,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T", [1, 8, 29])
+@pytest.mark.parametrize("T", [1, 8, 29, 300])
 @pytest.mark.parametrize("H,K,N,tail,dims,pad", [(4, 16, 40, 8, 8, 48), (3, 300, 7, 0, 0, 7), (20, 8, 150, 10, 6, 192),
-                                                 (2, 5, 11, 2, 2, 16)])
+                                                 (2, 5, 11, 2, 2, 16), (3, 72, 100, 24, 24, 128), (2, 136, 70, 0, 0, 70)])
 def test_products_per_head_with_gate_and_rotated_tail(dtype, T, H, K, N, tail, dims, pad):
     ops = _ops()
     from tffinfer_amd.parts.position import RotaryEmbedding
     g = torch.Generator().manual_seed(H * K + T)
     base = 300.0
-    x = torch.randn(T, 3 + H * (K + tail), generator=g).to(dtype)
-    wt = (torch.randn(H, K, N, generator=g) * 0.3).to(dtype)
+    lead = 8 if K % 8 == 0 else 3        # (aligned rows run on the matrix cores in bfloat16, others on the general kernel)
+    x = torch.randn(T, lead + H * (K + tail) + (-(lead + H * (K + tail))) % 8, generator=g).to(dtype)
+    wt = (torch.randn(H, N, K, generator=g) * 0.3).to(dtype)
     positions = torch.randint(0, 50, (T,), generator=g).to(torch.int32)
     table = RotaryEmbedding(tail, base, "interleaved", dims).table(64, DEV) if dims else None
-    out = ops.head_linear(x.to(DEV)[:, 3:], K + tail, wt.to(DEV), out_head=pad, tail=tail, cos_sin=table,
+    out = ops.head_linear(x.to(DEV)[:, lead:], K + tail, wt.to(DEV), out_head=pad, tail=tail, cos_sin=table,
                           positions=positions.to(DEV)).view(T, H, pad)
-    xh = x[:, 3:].double().view(T, H, K + tail)
-    ref = torch.einsum("thk,hkn->thn", xh[..., :K], wt.double())
+    xh = x[:, lead:lead + H * (K + tail)].double().view(T, H, K + tail)
+    ref = torch.einsum("thk,hnk->thn", xh[..., :K], wt.double())
     t_ = 3e-6 if dtype == torch.float32 else 8e-3
     assert _err(out[..., :N], ref) < t_
     if tail:
@@ -165,7 +177,7 @@ def test_products_per_head_with_gate_and_rotated_tail(dtype, T, H, K, N, tail, d
     if pad > N + tail:
         assert float(out[..., N + tail:].abs().max()) == 0
     gate = torch.randn(T, H * N + 4, generator=g).to(dtype)
-    gated = ops.head_linear(x.to(DEV)[:, 3:], K + tail, wt.to(DEV), gate=gate.to(DEV)[:, :H * N]).view(T, H, N)
+    gated = ops.head_linear(x.to(DEV)[:, lead:], K + tail, wt.to(DEV), gate=gate.to(DEV)[:, :H * N]).view(T, H, N)
     assert _err(gated, ref * torch.sigmoid(gate[:, :H * N].double().view(T, H, N))) < t_
 
 

@@ -11,10 +11,15 @@
 // page holds c in its first kv_rank rows and zeros below.
 //
 // tff_latent_kv_store:  c = rmsnorm(x[:rank]) * w, kr = rotate(x[rank:]) into the token's slot.
-// tff_head_linear:      out[t, h, :N] = x[t, h, :K] . Wt[h]  (Wt [H, K, N]), per head, with
+// tff_head_linear:      out[t, h, :N] = W[h] x[t, h, :K]  (W [H, N, K]), per head, with
 //                       an optional sigmoid gate on the result and an optional tail of the
 //                       input row that is rotated by the token's position and copied behind
 //                       the product (the query's rotated part), zeros up to pad_to.
+//                       bfloat16 on the matrix cores where rows are 16-byte aligned: a wave
+//                       holds 32 tokens x 64 outputs in accumulators and reads its operands
+//                       straight from memory in MFMA fragment order (eight consecutive k a
+//                       lane), W as the first operand so that a lane ends up with four
+//                       consecutive outputs of one token.
 #include "common.h"
 #include "tffinfer_kernels.h"
 
@@ -88,10 +93,10 @@ TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, in
 }
 
 // ---------------------------------------------------------------- per-head products ---
-// One block per (TT tokens, head, 256 output columns).  The block's input rows go to LDS as
-// float32, KC elements at a time; thread n walks k, reading Wt[h][k][n] (neighbouring threads,
-// neighbouring addresses) and adding into TT accumulators, k ascending for every token
-// whatever the batch.
+// The general kernel (float32, and bfloat16 rows that are not 16-byte aligned): one block per
+// (TT tokens, head, 256 output columns).  The block's input rows go to LDS as float32, KC
+// elements at a time; thread n walks k along its row W[h][n][:], adding into TT accumulators,
+// k ascending for every token whatever the batch.
 #define HL_TT 8
 #define HL_KC 128
 
@@ -104,6 +109,30 @@ struct HeadLinearTail {
     const int32_t* positions;      // per token
 };
 
+// The tail of the input heads of tokens t0 .. t0 + nt - 1 of head h, rotated and copied behind the
+// N products, zeros up to pad_to; by all threads of the block.
+template <typename T>
+__device__ __forceinline__ void head_tail(const T* __restrict__ x, int x_row, int x_head, T* __restrict__ out,
+                                          int out_row, int out_head, int t0, int nt, int h, int K, int N,
+                                          const HeadLinearTail tl) {
+    const int extra = tl.pad_to - N;
+    for (int i = threadIdx.x; i < nt * extra; i += blockDim.x) {
+        const int tt = i / extra, e = i - tt * extra;
+        const T* xr = x + (size_t)(t0 + tt) * x_row + (size_t)h * x_head + K;
+        float v = 0.f;
+        if (e < tl.tail) {
+            v = to_f32(xr[e]);
+            if (e < tl.rot_dims) {
+                const int pos = min(max(tl.positions[t0 + tt], 0), tl.max_pos - 1);
+                const float* cs = tl.cos_sin + ((size_t)pos * (tl.rot_dims >> 1) + (e >> 1)) * 2;
+                const float u = to_f32(xr[e & ~1]), w = to_f32(xr[e | 1]);
+                v = (e & 1) ? fmaf(w, cs[0], u * cs[1]) : fmaf(u, cs[0], -(w * cs[1]));
+            }
+        }
+        out[(size_t)(t0 + tt) * out_row + (size_t)h * out_head + N + e] = from_f32<T>(v);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void head_linear_kernel(
     const T* __restrict__ x, int x_row, int x_head, const T* __restrict__ Wt, T* __restrict__ out, int out_row,
@@ -112,7 +141,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
     const int t0 = blockIdx.x * HL_TT, h = blockIdx.y, tid = threadIdx.x;
     const int n = blockIdx.z * 256 + tid;
     const int nt = min(HL_TT, Tn - t0);
-    const T* W = Wt + (size_t)h * K * N;
+    const T* W = Wt + ((size_t)h * N + min(n, N - 1)) * K;      // the thread's row
     float acc[HL_TT];
 #pragma unroll
     for (int i = 0; i < HL_TT; ++i) acc[i] = 0.f;
@@ -126,7 +155,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
         __syncthreads();
         if (n < N) {
             for (int k = 0; k < kc; ++k) {
-                const float w = to_f32(W[(size_t)(k0 + k) * N + n]);
+                const float w = to_f32(W[k0 + k]);
 #pragma unroll
                 for (int i = 0; i < HL_TT; ++i) acc[i] = fmaf(xs[i][k], w, acc[i]);
             }
@@ -144,24 +173,87 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
             out[(size_t)(t0 + i) * out_row + (size_t)h * out_head + n] = from_f32<T>(v);
         }
     }
-    if (blockIdx.z == 0 && tl.pad_to > N) {
-        const int extra = tl.pad_to - N;
-        for (int i = tid; i < nt * extra; i += 256) {
-            const int tt = i / extra, e = i - tt * extra;
-            const T* xr = x + (size_t)(t0 + tt) * x_row + (size_t)h * x_head + K;
-            float v = 0.f;
-            if (e < tl.tail) {
-                v = to_f32(xr[e]);
-                if (e < tl.rot_dims) {
-                    const int pos = min(max(tl.positions[t0 + tt], 0), tl.max_pos - 1);
-                    const float* cs = tl.cos_sin + ((size_t)pos * (tl.rot_dims >> 1) + (e >> 1)) * 2;
-                    const float u = to_f32(xr[e & ~1]), w = to_f32(xr[e | 1]);
-                    v = (e & 1) ? fmaf(w, cs[0], u * cs[1]) : fmaf(u, cs[0], -(w * cs[1]));
+    if (blockIdx.z == 0 && tl.pad_to > N) head_tail<T>(x, x_row, x_head, out, out_row, out_head, t0, nt, h, K, N, tl);
+}
+
+// bfloat16 on the matrix cores.  Block: 128 tokens x 64 outputs of one head, four waves of 32
+// tokens each.  C[n][t] += W[n][k] x[t][k]: W's rows are the first operand's rows, so lane
+// (t = lane & 15, kg = lane >> 4) holds outputs n = kg * 4 .. + 3 of token t for each of the
+// 4 x 2 tiles.  k ascends in steps of 32 for every token whatever the batch.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hl_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hl_floatx4;
+
+__device__ __forceinline__ hl_bf16x8 hl_load8(const bf16_t* p, bool ok) {
+    union { uint4 u; hl_bf16x8 v; } x;
+    x.u = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
+    return x.v;
+}
+
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(
+    const bf16_t* __restrict__ x, int x_row, int x_head, const bf16_t* __restrict__ W, bf16_t* __restrict__ out,
+    int out_row, int out_head, int Tn, int K, int N, const bf16_t* __restrict__ gate, int gate_row,
+    HeadLinearTail tl) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, kg = lane >> 4;
+    const int h = blockIdx.y, n0 = blockIdx.z * 64;
+    const int tb = blockIdx.x * 128, t0 = tb + wv * 32;
+    hl_floatx4 acc[4][2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) acc[j][i] = hl_floatx4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* xp[2];
+    bool xok[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int t = t0 + i * 16 + r;
+        xok[i] = t < Tn;
+        xp[i] = x + (size_t)min(t, Tn - 1) * x_row + (size_t)h * x_head + kg * 8;
+    }
+    const bf16_t* wp[4];
+    bool wok[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + j * 16 + r;
+        wok[j] = n < N;
+        wp[j] = W + ((size_t)h * N + min(n, N - 1)) * K + kg * 8;
+    }
+    if (t0 < Tn) {      // (a wave's condition: the MFMAs below run for whole waves)
+        for (int k0 = 0; k0 < K; k0 += 32) {
+            const bool kok = k0 + kg * 8 < K;      // K is a multiple of 8: a lane's eight elements exist together
+            hl_bf16x8 a[4], b[2];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) a[j] = hl_load8(wp[j] + k0, wok[j] && kok);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) b[i] = hl_load8(xp[i] + k0, xok[i] && kok);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int t = t0 + i * 16 + r;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float v4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int n = n0 + j * 16 + kg * 4 + e;
+                    if (t < Tn && n < N) {
+                        float v = v4[e];
+                        if (gate) {
+                            const float gz = (float)gate[(size_t)t * gate_row + (size_t)h * N + n];
+                            v *= 1.0f / (1.0f + expf(-gz));
+                        }
+                        out[(size_t)t * out_row + (size_t)h * out_head + n] = (bf16_t)v;
+                    }
                 }
             }
-            out[(size_t)(t0 + tt) * out_row + (size_t)h * out_head + N + e] = from_f32<T>(v);
         }
     }
+    if (blockIdx.z == 0 && tl.pad_to > N)
+        head_tail<bf16_t>(x, x_row, x_head, out, out_row, out_head, tb, min(128, Tn - tb), h, K, N, tl);
 }
 
 TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt, void* out, int out_row, int out_head,
@@ -185,9 +277,17 @@ TFF_API int tff_head_linear(const void* x, int x_row, int x_head, const void* Wt
     if (dtype == TFF_F32)
         head_linear_kernel<float><<<grid, 256, 0, s>>>((const float*)x, x_row, x_head, (const float*)Wt, (float*)out, out_row,
                                                        out_head, T, K, N, (const float*)gate, gate_row, tl);
-    else if (dtype == TFF_BF16)
-        head_linear_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)Wt, (bf16_t*)out,
-                                                        out_row, out_head, T, K, N, (const bf16_t*)gate, gate_row, tl);
+    else if (dtype == TFF_BF16) {
+        const bool aligned = K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+                             ((uintptr_t)Wt % 16) == 0;
+        if (aligned)
+            head_linear_mfma_kernel<<<dim3((T + 127) / 128, H, (N + 63) / 64), 256, 0, s>>>(
+                (const bf16_t*)x, x_row, x_head, (const bf16_t*)Wt, (bf16_t*)out, out_row, out_head, T, K, N,
+                (const bf16_t*)gate, gate_row, tl);
+        else
+            head_linear_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)Wt, (bf16_t*)out,
+                                                            out_row, out_head, T, K, N, (const bf16_t*)gate, gate_row, tl);
+    }
     else
         return tff_fail("head_linear: unknown dtype %d", dtype);
     return tff_check_launch("head_linear");

@@ -194,3 +194,224 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
         return tff_fail("experts_down: unknown dtype %d", dtype);
     return tff_check_launch("experts_down");
 }
+
+// ------------------------------------------------------------- many tokens: by expert ---
+// With many tokens a step the (token, expert) pairs are dealt to their experts first: every
+// expert's pairs fill tiles of 32 rows (the last one padded), so that a tile's rows share the
+// expert's matrices and the products run on the matrix cores.  A pair's row is computed from
+// the pair alone, k ascending, whatever tile and place it lands in: the result does not depend
+// on what else the step holds, nor on the order the pairs were dealt in.
+//
+// tff_experts_sort:     tile_expert[tile], tile_rows[tile * 32 + i] = pair (token * top + k) or -1,
+//                       num_tiles[0]; one block.  At most pairs / 32 + E tiles.
+// tff_experts_gate_up_tiles / tff_experts_down_tiles: the two products per tile.  The down
+//                       product writes out[k][t][:] = wts[t][k] * Wd y: `top` planes that the
+//                       norm after the feed-forward adds up in the order of k.
+#define EXT_ROWS 32
+
+__global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __restrict__ idx, int pairs, int E,
+                                                            int max_tiles, int32_t* __restrict__ tile_expert,
+                                                            int32_t* __restrict__ tile_rows,
+                                                            int32_t* __restrict__ num_tiles) {
+    __shared__ int count[RT_MAX_E];
+    __shared__ int first[RT_MAX_E + 1];     // an expert's first tile
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < pairs; p += blockDim.x) atomicAdd(&count[idx[p]], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int t = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = t;
+            t += (count[e] + EXT_ROWS - 1) / EXT_ROWS;
+        }
+        first[E] = t;
+        num_tiles[0] = t;
+    }
+    __syncthreads();
+    const int tiles = first[E];
+    for (int e = tid; e < E; e += blockDim.x) {
+        for (int t = first[e]; t < first[e + 1]; ++t) tile_expert[t] = e;
+        count[e] = 0;
+    }
+    for (int i = tid; i < tiles * EXT_ROWS; i += blockDim.x) tile_rows[i] = -1;
+    __syncthreads();
+    for (int p = tid; p < pairs; p += blockDim.x) {
+        const int e = idx[p];
+        const int at = atomicAdd(&count[e], 1);
+        tile_rows[first[e] * EXT_ROWS + at] = p;
+    }
+}
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 ex_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ex_floatx4;
+
+__device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
+    union { uint4 u; ex_bf16x8 v; } x;
+    x.u = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
+    return x.v;
+}
+
+// Block: one tile of 32 pairs x 128 outputs, four waves of 32 outputs each (gate and up both).
+// C[f][pair] += W[f][k] h[pair][k]: lane (pair = lane & 15, kg = lane >> 4) ends up with outputs
+// f = kg * 4 .. + 3 of its pair.
+__global__ __launch_bounds__(256) void experts_gate_up_tiles_kernel(
+    const bf16_t* __restrict__ h, int h_row, const bf16_t* __restrict__ Wg, const bf16_t* __restrict__ Wu,
+    const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
+    const int32_t* __restrict__ num_tiles, int top, int width, int ff, float limit, float act_alpha,
+    bf16_t* __restrict__ y) {
+    const int tile = blockIdx.x;
+    if (tile >= num_tiles[0]) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, kg = lane >> 4;
+    const int e = tile_expert[tile];
+    const int f0 = blockIdx.y * 128 + wv * 32;
+    if (f0 >= ff) return;       // (a whole wave)
+    int pair[2];
+    const bf16_t* hp[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        pair[i] = tile_rows[tile * EXT_ROWS + i * 16 + r];
+        hp[i] = h + (size_t)(max(pair[i], 0) / top) * h_row + kg * 8;
+    }
+    const bf16_t *gp[2], *up[2];
+    bool fok[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int f = f0 + j * 16 + r;
+        fok[j] = f < ff;
+        gp[j] = Wg + ((size_t)e * ff + min(f, ff - 1)) * width + kg * 8;
+        up[j] = Wu + ((size_t)e * ff + min(f, ff - 1)) * width + kg * 8;
+    }
+    ex_floatx4 ag[2][2], au[2][2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) ag[j][i] = au[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < width; k0 += 32) {
+        const bool kok = k0 + kg * 8 < width;
+        ex_bf16x8 b[2], g[2], u[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) b[i] = ex_load8(hp[i] + k0, kok && pair[i] >= 0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            g[j] = ex_load8(gp[j] + k0, kok && fok[j]);
+            u[j] = ex_load8(up[j] + k0, kok && fok[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                ag[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g[j], b[i], ag[j][i], 0, 0, 0);
+                au[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[j], b[i], au[j][i], 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        if (pair[i] < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int f = f0 + j * 16 + kg * 4 + c;
+                if (f >= ff) continue;
+                const float gv = fminf(ag[j][i][c], limit);
+                const float uv = fminf(fmaxf(au[j][i][c], -limit), limit);
+                y[(size_t)pair[i] * ff + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
+            }
+    }
+}
+
+// Block: one tile of 32 pairs x 256 outputs of the width, four waves of 64 outputs each.
+__global__ __launch_bounds__(256) void experts_down_tiles_kernel(
+    const bf16_t* __restrict__ y, const bf16_t* __restrict__ Wd, const int32_t* __restrict__ tile_expert,
+    const int32_t* __restrict__ tile_rows, const int32_t* __restrict__ num_tiles, const float* __restrict__ wts,
+    int T, int top, int width, int ff, float* __restrict__ out) {
+    const int tile = blockIdx.x;
+    if (tile >= num_tiles[0]) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, kg = lane >> 4;
+    const int e = tile_expert[tile];
+    const int n0 = blockIdx.y * 256 + wv * 64;
+    if (n0 >= width) return;
+    int pair[2];
+    const bf16_t* yp[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        pair[i] = tile_rows[tile * EXT_ROWS + i * 16 + r];
+        yp[i] = y + (size_t)max(pair[i], 0) * ff + kg * 8;
+    }
+    const bf16_t* wp[4];
+    bool nok[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + j * 16 + r;
+        nok[j] = n < width;
+        wp[j] = Wd + ((size_t)e * width + min(n, width - 1)) * ff + kg * 8;
+    }
+    ex_floatx4 acc[4][2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < ff; k0 += 32) {
+        const bool kok = k0 + kg * 8 < ff;
+        ex_bf16x8 a[4], b[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) b[i] = ex_load8(yp[i] + k0, kok && pair[i] >= 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = ex_load8(wp[j] + k0, kok && nok[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        if (pair[i] < 0) continue;
+        const int t = pair[i] / top, k = pair[i] - t * top;
+        const float w = wts[pair[i]];
+        float* o = out + ((size_t)k * T + t) * width;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int n = n0 + j * 16 + kg * 4 + c;
+                if (n < width) o[n] = w * acc[j][i][c];
+            }
+    }
+}
+
+TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row) {
+    return width % 8 == 0 && ff % 8 == 0 && h_row % 8 == 0;
+}
+
+// h [T, width] bfloat16; workspace: tile_expert [max_tiles], tile_rows [max_tiles * 32], num_tiles [1] (int32),
+// y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 32 + E.
+TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
+                                 const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
+                                 float limit, float act_alpha, int32_t* tile_expert, int32_t* tile_rows,
+                                 int32_t* num_tiles, int max_tiles, void* y, float* out, tff_stream_t stream) {
+    TFF_REQUIRE(h && Wg && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
+                "experts_by_tiles: null pointer");
+    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= RT_MAX_E && width > 0 && ff > 0 && h_row >= width,
+                "experts_by_tiles: bad sizes T=%d top=%d E=%d width=%d ff=%d", T, top, E, width, ff);
+    TFF_REQUIRE(tff_experts_tiles_supported(width, ff, h_row), "experts_by_tiles: width %d, ff %d and rows of %d must be "
+                "multiples of 8", width, ff, h_row);
+    TFF_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0 &&
+                ((uintptr_t)Wd % 16) == 0 && ((uintptr_t)y % 16) == 0, "experts_by_tiles: operands must be 16-byte aligned");
+    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles >= (long)T * top / EXT_ROWS + E,
+                "experts_by_tiles: %d tiles do not hold %d x %d pairs of %d experts", max_tiles, T, top, E);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, max_tiles, tile_expert, tile_rows, num_tiles);
+    int rc = tff_check_launch("experts_sort");
+    if (rc) return rc;
+    experts_gate_up_tiles_kernel<<<dim3(max_tiles, (ff + 127) / 128), 256, 0, s>>>(
+        (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows, num_tiles, top, width, ff,
+        limit, act_alpha, (bf16_t*)y);
+    rc = tff_check_launch("experts_gate_up_tiles");
+    if (rc) return rc;
+    experts_down_tiles_kernel<<<dim3(max_tiles, (width + 255) / 256), 256, 0, s>>>(
+        (const bf16_t*)y, (const bf16_t*)Wd, tile_expert, tile_rows, num_tiles, wts, T, top, width, ff, out);
+    return tff_check_launch("experts_down_tiles");
+}

@@ -234,7 +234,7 @@ TFF_API int tff_latent_kv_store(const void* x, int x_stride, int T, int rank, in
                                 const float* norm_w, float eps, const float* cos_sin, int max_pos,
                                 const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache,
                                 int page_size, int num_pages, int Dp, int dtype, tff_stream_t stream);
-// Products per head: out[t, h * out_head + n] = sum_k x[t, h * x_head + k] * Wt[h, k, n], Wt [H, K, N].
+// Products per head: out[t, h * out_head + n] = sum_k x[t, h * x_head + k] * Wt[h, n, k], Wt [H, N, K].
 // gate (may be null): the result is multiplied by sigmoid(gate[t, h * N + n]).  tail > 0: the
 // `tail` elements of the input head behind the K multiplied ones are copied behind the N results,
 // the first rot_dims of them rotated in pairs (2i, 2i+1) by the token's position; pad_to > N + tail:
@@ -266,6 +266,17 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
 // out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff]; out float32.
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
                              int width, int ff, float* out, int dtype, tff_stream_t stream);
+
+// The same for steps of many tokens (bfloat16; width, ff and h_row multiples of 8): the (token, expert) pairs
+// are dealt to their experts in tiles of 32 rows and the two products run on the matrix cores.  out is
+// float32 [top, T, width], plane k = wts[:, k] * (expert k's output): the consumer adds the planes in order.
+// Workspace: tile_expert [max_tiles], tile_rows [32 * max_tiles], num_tiles [1], y [T * top, ff] bfloat16;
+// max_tiles >= T * top / 32 + E.
+TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row);
+TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
+                                 const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
+                                 float limit, float act_alpha, int32_t* tile_expert, int32_t* tile_rows,
+                                 int32_t* num_tiles, int max_tiles, void* y, float* out, tff_stream_t stream);
 
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

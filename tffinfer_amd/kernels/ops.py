@@ -944,7 +944,7 @@ def head_linear(x: torch.Tensor, x_head: int, weight_t: torch.Tensor, out_head: 
                 gate: torch.Tensor | None = None, tail: int = 0, cos_sin: torch.Tensor | None = None,
                 positions: torch.Tensor | None = None) -> torch.Tensor:
     """Products per head: x [T, >= H * x_head] (head h starts at h * x_head; rows may be strided),
-    ``weight_t`` [H, K, N]: out[t, h, :N] = x[t, h, :K] . weight_t[h].  Returns [T, H * out_head]
+    ``weight_t`` [H, N, K]: out[t, h, :N] = weight_t[h] x[t, h, :K].  Returns [T, H * out_head]
     (``out_head`` >= N + tail, by default N + tail), zeros behind what is written.
     ``gate`` [T, >= H * N] (rows may be strided): the products are multiplied by its sigmoid.
     ``tail``: so many elements of the input head behind the K are copied behind the products, the
@@ -952,7 +952,7 @@ def head_linear(x: torch.Tensor, x_head: int, weight_t: torch.Tensor, out_head: 
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise _lib.KernelError("head_linear x: expected a GPU matrix with unit inner stride")
     _req(weight_t, "head_linear weight", x.dtype, 3)
-    H, K, N = weight_t.shape
+    H, N, K = weight_t.shape
     T = x.shape[0]
     if x_head < K + tail or x.shape[1] < (H - 1) * x_head + K + tail:
         raise _lib.KernelError(f"head_linear: rows of {x.shape[1]} do not hold {H} heads of {K} + {tail}, {x_head} apart")
@@ -1038,11 +1038,19 @@ def route_topk(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None,
     return idx, wts
 
 
+#: tokens from which a step's (token, expert) pairs are dealt to their experts and run on the matrix
+#: cores; below, every pair streams its expert's rows itself, which is what few tokens are bound by
+EXPERT_TILES_MIN_TOKENS = 32
+
+
 def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                   idx: torch.Tensor, wts: torch.Tensor, limit: float, act_alpha: float) -> torch.Tensor:
+                   idx: torch.Tensor, wts: torch.Tensor, limit: float, act_alpha: float,
+                   by_tiles: bool | None = None) -> torch.Tensor:
     """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + 1) with
     g = min(Wg h, limit), u = clamp(Wu h, -limit, limit); out = sum_k wts[:, k] Wd y.
-    ``w_gate``, ``w_up`` [E, ff, width], ``w_down`` [E, width, ff] of h's type; float32 [T, width]."""
+    ``w_gate``, ``w_up`` [E, ff, width], ``w_down`` [E, width, ff] of h's type.  float32
+    [T, width], or (many tokens in bfloat16, ``by_tiles``) [top, T, width]: the terms of the sum
+    over k, which ``scale_add_rmsnorm`` and ``as_tensor`` add up in order."""
     _req(h, "routed_experts h", ndim=2)
     T, width = h.shape
     for w, nm in ((w_gate, "gate"), (w_up, "up"), (w_down, "down")):
@@ -1059,6 +1067,19 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
         raise _lib.KernelError("routed_experts: idx and weights must be [T, top]")
     L = _lib.load()
     y = torch.empty(T * top, ff, dtype=h.dtype, device=h.device)
+    if by_tiles is None:
+        by_tiles = T >= EXPERT_TILES_MIN_TOKENS
+    if by_tiles and h.dtype == torch.bfloat16 and L.tff_experts_tiles_supported(width, ff, width):
+        # many tokens: the pairs dealt to their experts, the products on the matrix cores; the result
+        # comes as one plane per chosen expert, for the norm that follows to add up in their order
+        max_tiles = T * top // 32 + E
+        tables = torch.empty(33 * max_tiles + 1, dtype=torch.int32, device=h.device)
+        out = torch.empty(top, T, width, dtype=torch.float32, device=h.device)
+        _lib.check(L.tff_experts_by_tiles(
+            h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+            T, top, E, width, ff, float(limit), float(act_alpha), tables.data_ptr(), tables[max_tiles:].data_ptr(),
+            tables[33 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
+        return out if top > 1 else out[0]
     _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), idx.data_ptr(), T, top, E,
                                      width, ff, float(limit), float(act_alpha), y.data_ptr(), dtype_code(h.dtype), _stream()))
     out = torch.empty(T, width, dtype=torch.float32, device=h.device)

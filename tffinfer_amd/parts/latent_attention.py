@@ -99,10 +99,10 @@ class LatentAttention(Mixer):
         stacked = [weights["q"], weights["dkv"]] + ([weights["g"]] if self.has_gate else [])
         self.w_in = to_device(torch.cat([w.to(stacked[0].dtype) for w in stacked], 0), dtype, device)
         self.w_o = to_device(weights["o"], dtype, device)
-        # [H, head_dim, rank]: k_h^n = Wuk_h c, so (Wuk_h^T q)[r] = sum_d q[d] Wuk[h, d, r]
-        self.w_uk_t = weights["uk"].to(dtype).view(H, self.head_dim, self.kv_rank).contiguous().to(device)
-        # [H, rank, value_dim]: v_h[e] = sum_r Wuv[h, e, r] c[r]
-        self.w_uv_t = weights["uv"].to(dtype).view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous().to(device)
+        # per head [outputs, inputs]: k_h^n = Wuk_h c, so (Wuk_h^T q)[r] = sum_d Wuk[h, d, r] q[d]: [H, rank, head_dim]
+        self.w_uk_t = weights["uk"].to(dtype).view(H, self.head_dim, self.kv_rank).transpose(1, 2).contiguous().to(device)
+        # v_h[e] = sum_r Wuv[h, e, r] c[r]: [H, value_dim, rank], as stored
+        self.w_uv_t = weights["uv"].to(dtype).view(H, self.value_dim, self.kv_rank).contiguous().to(device)
         self.latent_norm = weights["dkv.norm"].to(torch.float32).contiguous().to(device)
         self.sink = weights["sink"].to(torch.float32).contiguous().to(device) if self.has_sink else None
 
