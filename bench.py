@@ -34,6 +34,81 @@ SHAPES = {
 }
 
 
+
+
+def disunex_shape(width, heads, dim, rot, vdim, rank, window, dense_ff, experts, top, expert_ff, layers, vocab=151936):
+    """A Disunex configuration of ``layers`` layers, dense and routed feed-forwards in turn."""
+    mix = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+           "mask": {"size": window}, "rot": {"base": 1000000.0, "dims": rot}}
+    mlps = [{"kind": "dense", "ff": dense_ff},
+            {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}]
+    return {"architecture": "Disunex", "width": width, "vocab": vocab, "postln_alpha": 1.0, "norm": {"eps": 1e-6},
+            "layers": [{"type": "latent_attention", "mixer": mix, "mlp": mlps[i % 2]} for i in range(layers)]}
+
+
+# Disunex at sizes that resemble a real model's layers, each beside the Qwen3 shape of the same width
+# (per layer about as many matrix elements a token: the dense feed-forward has two matrices where the
+# gated one has three, so it is half again as wide)
+DISUNEX_SHAPES = {
+    "2k": ("1.7b", dict(width=2048, heads=16, dim=64, rot=32, vdim=64, rank=96, window=1024, dense_ff=9216,
+                        experts=16, top=2, expert_ff=1024)),
+    "4k": ("8b", dict(width=4096, heads=32, dim=128, rot=64, vdim=128, rank=192, window=1024, dense_ff=18432,
+                      experts=32, top=4, expert_ff=1536)),
+}
+
+
+def design_points(args):
+    """Prefill and decode throughput of the Disunex design at the sizes of DISUNEX_SHAPES, and of the
+    Qwen3 shape of the same width and number of layers beside it, one JSON line."""
+    import gc
+    import torch
+    from tffinfer_amd import EngineOptions, LLMEngine
+    from tffinfer_amd import measure as M
+    from tffinfer_amd.kernels import lib as kernel_lib
+    kernel_lib.load()
+    gen = torch.Generator().manual_seed(args.seed)
+    L = args.layers or 8
+    T, batch, context = args.prefill_tokens, args.batch, args.context
+    steps, warmup = min(args.steps, 32), min(args.warmup, 4)
+    out = {"design": "Disunex", "layers_run": L, "prefill_tokens": T, "decode_batch": batch, "decode_context": context,
+           "dtype": "bf16", "data": "synthetic (seeded random weights and token ids)", "shapes": {}}
+    which = [args.design_shape] if args.design_shape else sorted(DISUNEX_SHAPES)
+    for name in which:
+        beside, sizes = DISUNEX_SHAPES[name]
+        row = {}
+        for label, cfg in (("disunex", disunex_shape(layers=L, **sizes)),
+                           ("qwen3_" + beside, dict(SHAPES[beside][1], num_hidden_layers=L))):
+            if args.design_only and label != args.design_only and not label.startswith(args.design_only):
+                continue
+            model = build_model(dict(cfg), args.seed)
+            vocab = model.config.vocab_size
+            total = steps + warmup + M.decode_slack(batch, context) + 16
+            opt = EngineOptions(dtype="bfloat16", page_size=args.page_size,
+                                kv_tokens=batch * (context + total + args.page_size) + T, max_num_seqs=batch,
+                                max_num_batched_tokens=max(4096, T), prefill_chunk=max(2048, T),
+                                max_model_len=max(T, context + total) + 16, use_graphs=not args.no_graphs)
+            engine = LLMEngine(model, opt)
+            r = {}
+            if args.only != "decode":
+                pre = M.measure_prefill(engine, gen, T, vocab)
+                flops = M.prefill_flops(model, T)
+                r.update(prefill_ms=round(1e3 * pre["wall_s"], 3), prefill_tokens_per_s=round(T / pre["wall_s"], 1),
+                         prefill_frac_of_bf16_peak=round(flops / pre["wall_s"] / M.MFMA_PEAK["bf16"], 4))
+            if args.only != "prefill":
+                dec = M.measure_decode(engine, gen, batch, context, steps, warmup, vocab)
+                step = dec["wall_s"] / steps
+                nbytes = M.decode_bytes(model, batch, context + warmup + steps / 2.0)
+                r.update(decode_ms_per_step=round(1e3 * step, 4), decode_tokens_per_s=round(batch / step, 1),
+                         decode_frac_of_hbm_peak=round(nbytes / step / 1e9 / M.HBM_PEAK_GBS, 4))
+            r["matrix_elements_per_token_per_layer"] = M.matrix_elements_per_step(model) // L
+            row[label] = r
+            del engine, model
+            gc.collect()
+            torch.cuda.empty_cache()
+        out["shapes"][name] = row
+    print(json.dumps(out))
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,6 +139,12 @@ def parse_args():
                     help="with --mixed: the scheduler cuts steps a little over a multiple of this many tokens down "
                          "to the multiple (default: the engine's own, 256; 0: off)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--design", choices=["disunex"], default=None,
+                    help="instead of the benchmark line: prefill (--prefill-tokens) and decode (--batch, --context) "
+                         "throughput of this design at sizes that resemble a real model's layers, each beside the "
+                         "Qwen3 shape of the same width, --layers layers each (default 8)")
+    ap.add_argument("--design-shape", default=None, help="with --design: one of its sizes only (2k, 4k)")
+    ap.add_argument("--design-only", default=None, help="with --design: 'disunex' or 'qwen3' only (for profiling)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
                          "on this machine and stop")
@@ -201,6 +282,9 @@ def main():
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single GPU)")
         sys.exit(2)
+    if args.design:
+        design_points(args)
+        return
     import torch
     from tffinfer_amd import EngineOptions, LLMEngine
     from tffinfer_amd import measure as M

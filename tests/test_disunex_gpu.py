@@ -79,6 +79,11 @@ def test_router_choice_goes_by_the_corrected_scores_and_weights_by_the_plain_one
     assert torch.allclose(w.sum(-1).cpu(), torch.ones(T), atol=1e-5)
     idx0, _ = ops.route_topk(h.to(DEV), router.to(DEV), None, top)
     assert torch.equal(idx0.cpu().long(), plain_idx)
+    # the logits from the engine's own product: a bfloat16 router times bfloat16 rows is exact in float32
+    w_dev = router.to(dtype).to(DEV)
+    z = ops.linear(h.to(DEV), ops.pack_weight(w_dev) if dtype == torch.bfloat16 else w_dev, out_dtype=torch.float32)
+    idx1, w1 = ops.route_topk(None, None, corr.to(DEV), top, logits=z)
+    assert torch.equal(idx1.cpu().long(), ref_idx) and _err(w1, ref_w) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

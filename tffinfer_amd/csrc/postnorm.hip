@@ -65,6 +65,80 @@ __global__ __launch_bounds__(PN_THREADS) void scale_add_rmsnorm_kernel(
     }
 }
 
+// The same for rows whose width is a multiple of 4: 16-byte accesses; NT threads a row (1024 where
+// there are few rows: more loads in flight for each), rows of up to 4096 elements in registers.
+template <typename TO>
+__device__ __forceinline__ void pn_store4(TO* o, float4 v);
+template <>
+__device__ __forceinline__ void pn_store4<float>(float* o, float4 v) { *reinterpret_cast<float4*>(o) = v; }
+template <>
+__device__ __forceinline__ void pn_store4<bf16_t>(bf16_t* o, float4 v) {
+    union { bf16_t h[4]; uint2 u; } pk;
+    pk.h[0] = (bf16_t)v.x; pk.h[1] = (bf16_t)v.y; pk.h[2] = (bf16_t)v.z; pk.h[3] = (bf16_t)v.w;
+    *reinterpret_cast<uint2*>(o) = pk.u;
+}
+
+template <typename TO, int NT>
+__global__ __launch_bounds__(NT) void scale_add_rmsnorm_vec_kernel(
+    float* __restrict__ resid, const float* __restrict__ delta, int planes, size_t plane, float alpha,
+    const float* __restrict__ w, float eps, TO* __restrict__ out, int H) {
+    __shared__ float red[17];
+    constexpr int ITS = 1024 / NT;
+    const int r = blockIdx.x, tid = threadIdx.x, H4 = H >> 2;
+    const size_t plane4 = plane >> 2;
+    float4* x4 = reinterpret_cast<float4*>(resid + (size_t)r * H);
+    const float4* d4 = delta ? reinterpret_cast<const float4*>(delta + (size_t)r * H) : nullptr;
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    auto sum_at = [&](int j) {
+        float4 v = x4[j];
+        v.x *= alpha; v.y *= alpha; v.z *= alpha; v.w *= alpha;
+        if (d4) {
+            float4 d = d4[j];
+            for (int p = 1; p < planes; ++p) {
+                const float4 e = d4[(size_t)p * plane4 + j];
+                d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+            }
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        return v;
+    };
+    float4 cache[ITS];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        const int j = tid + it * NT;
+        if (j < H4) {
+            const float4 v = sum_at(j);
+            cache[it] = v;
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+        }
+    }
+    for (int j = tid + 1024; j < H4; j += NT) {
+        const float4 v = sum_at(j);
+        x4[j] = v;      // (kept in place for the second sweep)
+        ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+    }
+    ss = block_sum(ss, red);
+    const float rr = 1.0f / sqrtf(ss / (float)H + eps);
+    TO* o = out ? out + (size_t)r * H : nullptr;
+#pragma unroll
+    for (int it = 0; it < ITS; ++it) {
+        const int j = tid + it * NT;
+        if (j < H4) {
+            const float4 v = cache[it], wv = w4[j];
+            const float4 y = make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w);
+            x4[j] = y;
+            if (o) pn_store4<TO>(o + 4 * j, y);
+        }
+    }
+    for (int j = tid + 1024; j < H4; j += NT) {
+        const float4 v = x4[j], wv = w4[j];
+        const float4 y = make_float4(v.x * rr * wv.x, v.y * rr * wv.y, v.z * rr * wv.z, v.w * rr * wv.w);
+        x4[j] = y;
+        if (o) pn_store4<TO>(o + 4 * j, y);
+    }
+}
+
 TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_planes, size_t delta_plane, float alpha,
                                   const float* weight, float eps, void* out, int n, int H, int out_dtype,
                                   tff_stream_t stream) {
@@ -75,6 +149,20 @@ TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_pl
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const int planes = delta ? delta_planes : 0;
+    const bool vec = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)weight % 16) == 0 &&
+                     (!out || ((uintptr_t)out % 16) == 0) &&
+                     (!delta || (((uintptr_t)delta % 16) == 0 && (planes == 1 || delta_plane % 4 == 0)));
+    if (vec) {
+        const bool wide = n <= 128 && H >= 2048;
+        if (out_dtype == TFF_F32) {
+            if (wide) scale_add_rmsnorm_vec_kernel<float, 1024><<<n, 1024, 0, s>>>(resid, delta, planes, delta_plane, alpha, weight, eps, (float*)out, H);
+            else scale_add_rmsnorm_vec_kernel<float, 256><<<n, 256, 0, s>>>(resid, delta, planes, delta_plane, alpha, weight, eps, (float*)out, H);
+        } else {
+            if (wide) scale_add_rmsnorm_vec_kernel<bf16_t, 1024><<<n, 1024, 0, s>>>(resid, delta, planes, delta_plane, alpha, weight, eps, (bf16_t*)out, H);
+            else scale_add_rmsnorm_vec_kernel<bf16_t, 256><<<n, 256, 0, s>>>(resid, delta, planes, delta_plane, alpha, weight, eps, (bf16_t*)out, H);
+        }
+        return tff_check_launch("scale_add_rmsnorm");
+    }
     if (out_dtype == TFF_F32)
         scale_add_rmsnorm_kernel<float><<<n, PN_THREADS, 0, s>>>(resid, delta, planes, delta_plane, alpha, weight, eps,
                                                                  (float*)out, H);

@@ -1,6 +1,6 @@
 // A feed-forward made of many small experts of which every token uses a few.
 //
-// tff_route_topk:   z = Wr h in float32, s = sigmoid(z); the `top` experts with the largest
+// tff_route_topk:   z = Wr h in float32 (or given: a product that ran before), s = sigmoid(z); the `top` experts with the largest
 //                   s + bias are chosen (the lowest index among equals), their weights are
 //                   s / (sum of the chosen s + 1e-20): the bias moves the choice only.
 // tff_experts_gate_up: for every (token, chosen expert): g = min(Wg h, limit),
@@ -45,24 +45,40 @@ __device__ __forceinline__ float row_dot<bf16_t>(const bf16_t* a, const bf16_t* 
 
 #define RT_MAX_E 1024
 
+// One block of RT_WAVES waves per token.  logits != null: z is given (a product that ran before);
+// else the waves compute it, each its share of the experts, 16 bytes a lane and load.
+#define RT_WAVES 8
+
 template <typename T>
-__global__ __launch_bounds__(64) void route_topk_kernel(const T* __restrict__ h, int h_row, const float* __restrict__ Wr,
-                                                        const float* __restrict__ bias, int width, int E, int top,
-                                                        int32_t* __restrict__ idx, float* __restrict__ wts) {
+__global__ __launch_bounds__(64 * RT_WAVES) void route_topk_kernel(const T* __restrict__ h, int h_row,
+                                                                   const float* __restrict__ Wr,
+                                                                   const float* __restrict__ logits,
+                                                                   const float* __restrict__ bias, int width, int E,
+                                                                   int top, int32_t* __restrict__ idx,
+                                                                   float* __restrict__ wts) {
     __shared__ float s_all[RT_MAX_E];
     __shared__ float c_all[RT_MAX_E];
     __shared__ int chosen[64];
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const T* hr = h + (size_t)t * h_row;
-    for (int e = 0; e < E; ++e) {
-        const float z = wave_dot(hr, Wr + (size_t)e * width, width, lane);
-        if (lane == 0) {
-            const float s = 1.0f / (1.0f + expf(-z));
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (logits) {
+        for (int e = threadIdx.x; e < E; e += blockDim.x) {
+            const float s = 1.0f / (1.0f + expf(-logits[(size_t)t * E + e]));
             s_all[e] = s;
             c_all[e] = s + (bias ? bias[e] : 0.f);
         }
+    } else {
+        const T* hr = h + (size_t)t * h_row;
+        for (int e = wv; e < E; e += RT_WAVES) {
+            const float z = wave_dot(hr, Wr + (size_t)e * width, width, lane);
+            if (lane == 0) {
+                const float s = 1.0f / (1.0f + expf(-z));
+                s_all[e] = s;
+                c_all[e] = s + (bias ? bias[e] : 0.f);
+            }
+        }
     }
     __syncthreads();
+    if (wv > 0) return;
     float sum = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
@@ -77,31 +93,32 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const T* __restrict__ h,
             const int oi = __shfl_xor(bi, o, 64);
             if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
         }
-        __syncthreads();
+        // (one wave from here on: LDS works through its accesses in order)
         if (lane == 0) {
             idx[(size_t)t * top + k] = bi;
             chosen[k] = bi;
             c_all[bi] = -INFINITY;
         }
         sum += s_all[bi];
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        __builtin_amdgcn_wave_barrier();
     }
     const float inv = 1.0f / (sum + 1e-20f);
     if (lane < top) wts[(size_t)t * top + lane] = s_all[chosen[lane]] * inv;
 }
 
-TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* bias, int T, int width, int E,
-                           int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream) {
-    TFF_REQUIRE(h && Wr && idx && wts, "route_topk: null pointer");
-    TFF_REQUIRE(T >= 0 && width > 0 && h_row >= width, "route_topk: bad sizes T=%d width=%d row=%d", T, width, h_row);
+TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
+                           int width, int E, int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream) {
+    TFF_REQUIRE(idx && wts && (logits || (h && Wr)), "route_topk: null pointer");
+    TFF_REQUIRE(T >= 0 && (logits || (width > 0 && h_row >= width)), "route_topk: bad sizes T=%d width=%d row=%d", T, width, h_row);
     TFF_REQUIRE(E > 0 && E <= RT_MAX_E && top > 0 && top <= E && top <= 64,
                 "route_topk: %d of %d experts (up to 64 of up to %d)", top, E, RT_MAX_E);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TFF_F32)
-        route_topk_kernel<float><<<T, 64, 0, s>>>((const float*)h, h_row, Wr, bias, width, E, top, idx, wts);
+        route_topk_kernel<float><<<T, 64 * RT_WAVES, 0, s>>>((const float*)h, h_row, Wr, logits, bias, width, E, top, idx, wts);
     else if (dtype == TFF_BF16)
-        route_topk_kernel<bf16_t><<<T, 64, 0, s>>>((const bf16_t*)h, h_row, Wr, bias, width, E, top, idx, wts);
+        route_topk_kernel<bf16_t><<<T, 64 * RT_WAVES, 0, s>>>((const bf16_t*)h, h_row, Wr, logits, bias, width, E, top, idx, wts);
     else
         return tff_fail("route_topk: unknown dtype %d", dtype);
     return tff_check_launch("route_topk");

@@ -254,10 +254,11 @@ TFF_API int tff_scale_add_rmsnorm(float* resid, const float* delta, int delta_pl
 TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dtype, tff_stream_t stream);
 
 // ---- routed experts (routed_experts.hip) ----
-// Router: s = sigmoid(Wr h) in float32 (Wr [E, width] float32); the `top` largest s + bias (bias may
-// be null) are chosen; idx [T, top], wts [T, top] = s / (sum of the chosen s + 1e-20).
-TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* bias, int T, int width, int E,
-                           int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
+// Router: s = sigmoid(z), z = Wr h in float32 (Wr [E, width] float32), or z = logits [T, E] where given
+// (h and Wr may then be null); the `top` largest s + bias (bias may be null) are chosen; idx [T, top],
+// wts [T, top] = s / (sum of the chosen s + 1e-20).
+TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
+                           int width, int E, int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
 // y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + 1), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
 // e = idx[t, k]; Wg, Wu [E, ff, width].
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,

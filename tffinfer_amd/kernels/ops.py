@@ -1018,23 +1018,32 @@ def gelu(x: torch.Tensor, tanh_form: bool = False) -> torch.Tensor:
     return out
 
 
-def route_topk(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int):
-    """s = sigmoid(h . router^T) in float32 (router float32 [E, width]); the ``top`` experts with
-    the largest s + bias; returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20))."""
-    _req(h, "route_topk h", ndim=2)
-    _req(router, "router", torch.float32, 2)
-    T, width = h.shape
-    E = router.shape[0]
-    if router.shape[1] != width:
-        raise _lib.KernelError(f"route_topk: router {tuple(router.shape)} for rows of {width}")
+def route_topk(h: torch.Tensor | None, router: torch.Tensor | None, bias: torch.Tensor | None, top: int,
+               logits: torch.Tensor | None = None):
+    """s = sigmoid(z) with z = h . router^T in float32 (router float32 [E, width]) or z = ``logits``
+    (float32 [T, E], a product that ran before); the ``top`` experts with the largest s + bias;
+    returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20))."""
+    if logits is not None:
+        _req(logits, "router logits", torch.float32, 2)
+        T, E = logits.shape
+        width, dev, dt = 0, logits.device, torch.float32
+    else:
+        _req(h, "route_topk h", ndim=2)
+        _req(router, "router", torch.float32, 2)
+        T, width = h.shape
+        E = router.shape[0]
+        dev, dt = h.device, h.dtype
+        if router.shape[1] != width:
+            raise _lib.KernelError(f"route_topk: router {tuple(router.shape)} for rows of {width}")
     if bias is not None:
         _req(bias, "router bias", torch.float32, 1)
         if bias.numel() != E:
             raise _lib.KernelError(f"route_topk: {bias.numel()} bias terms for {E} experts")
-    idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
-    wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
-    _lib.check(_lib.load().tff_route_topk(h.data_ptr(), width, router.data_ptr(), _ptr(bias), T, width, E, int(top),
-                                          idx.data_ptr(), wts.data_ptr(), dtype_code(h.dtype), _stream()))
+    idx = torch.empty(T, top, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, top, dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().tff_route_topk(None if logits is not None else h.data_ptr(), width,
+                                          None if logits is not None else router.data_ptr(), _ptr(logits), _ptr(bias),
+                                          T, width, E, int(top), idx.data_ptr(), wts.data_ptr(), dtype_code(dt), _stream()))
     return idx, wts
 
 

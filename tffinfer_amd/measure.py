@@ -21,17 +21,22 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
 
 
-def _matrix_elements(part) -> int:
-    """Elements of the matrices a part and its sub-parts multiply with."""
+def _matrix_elements(part, rows: int = 1, streamed: bool = False) -> int:
+    """Elements of the matrices a part and its sub-parts multiply a token's row with (a part
+    that uses only some of its matrices for a token says how many: ``active_matrix_elements``),
+    or, ``streamed``, the elements a step of ``rows`` tokens has to read (``streamed_matrix_elements``)."""
+    own = getattr(part, "streamed_matrix_elements" if streamed else "active_matrix_elements", None)
+    if own is not None:
+        return own(rows) if streamed else own()
     n = sum(math.prod(spec.shape) for spec in part.weight_specs().values()
             if spec.init == "matrix" and len(spec.shape) == 2)
-    return n + sum(_matrix_elements(child) for child in part.children().values())
+    return n + sum(_matrix_elements(child, rows, streamed) for child in part.children().values())
 
 
-def matrix_elements_per_step(model) -> int:
-    """Elements of all matrices a step multiplies a token's row with, a layer that the run order
-    names twice counted twice; without the output head."""
-    return sum(_matrix_elements(model.blocks[call.layer]) for call in model.schedule)
+def matrix_elements_per_step(model, rows: int = 1, streamed: bool = False) -> int:
+    """Elements of all matrices a step multiplies a token's row with (or, ``streamed``, reads for
+    ``rows`` tokens), a layer that the run order names twice counted twice; without the output head."""
+    return sum(_matrix_elements(model.blocks[call.layer], rows, streamed) for call in model.schedule)
 
 
 def prefill_flops(model, T: int) -> float:
@@ -57,7 +62,7 @@ def decode_bytes(model, batch: int, context: float, esz: int = 2) -> float:
     with once (a layer that the run order names twice, twice), the output head, and the keys and
     values that every layer call reads for the live requests (a window's worth where it has one)."""
     cfg = model.config
-    weights = (matrix_elements_per_step(model) + cfg.hidden_size * cfg.vocab_size) * esz
+    weights = (matrix_elements_per_step(model, batch, streamed=True) + cfg.hidden_size * cfg.vocab_size) * esz
     kv = 0.0
     for call in model.schedule:
         spec = model.blocks[call.layer].mixer.cache_spec()

@@ -121,7 +121,7 @@ class RoutedExperts(FeedForward):
         if not 0 < self.top <= self.num_experts:
             from ..config.base import ConfigError
             raise ConfigError(f"routed experts: top={self.top} of {self.num_experts} experts")
-        self.w_gate = self.w_up = self.w_down = self.router = self.correction = None
+        self.w_gate = self.w_up = self.w_down = self.router = self.router_w = self.correction = None
 
     def weight_specs(self):
         H, I = self.hidden_size, self.intermediate_size
@@ -139,6 +139,12 @@ class RoutedExperts(FeedForward):
         H, I = self.hidden_size, self.intermediate_size
         return self.num_experts * H + self.top * 3 * H * I
 
+    def streamed_matrix_elements(self, rows: int) -> int:
+        """Matrix elements a step of ``rows`` tokens reads at least: the router and as many
+        experts as the tokens can choose between them."""
+        H, I = self.hidden_size, self.intermediate_size
+        return self.num_experts * H + min(self.num_experts, rows * self.top) * 3 * H * I
+
     def load_weights(self, weights, dtype, device):
         E = self.num_experts
 
@@ -146,12 +152,23 @@ class RoutedExperts(FeedForward):
             return torch.stack([weights[f"e{e}.{which}"].to(dtype) for e in range(E)], 0).contiguous().to(device)
 
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
-        self.router = weights["router"].to(torch.float32).contiguous().to(device)
+        # The router's logits are float32 sums.  A router stored in bfloat16 multiplies exactly with
+        # bfloat16 rows on the matrix cores (the products of two bfloat16 numbers are float32 numbers,
+        # the sums are float32): the engine's own product serves.  One stored in more bits keeps them,
+        # and the routing kernel forms the logits itself.
+        self.router_w = None
+        if dtype == torch.float32 or weights["router"].dtype == torch.bfloat16:
+            self.router_w = to_device(weights["router"], dtype, device)
+        self.router = weights["router"].to(torch.float32).contiguous().to(device) if self.router_w is None else None
         self.correction = (weights["correction"].to(torch.float32).contiguous().to(device)
                            if self.has_correction else None)
 
     def forward(self, ctx, x):
         ops = ctx.ops
         x = ops.as_tensor(x)
-        idx, wts = ops.route_topk(x, self.router, self.correction, self.top)
+        if self.router_w is not None:
+            idx, wts = ops.route_topk(None, None, self.correction, self.top,
+                                      logits=ops.linear(x, self.router_w, out_dtype=torch.float32))
+        else:
+            idx, wts = ops.route_topk(x, self.router, self.correction, self.top)
         return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha)
