@@ -214,17 +214,17 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 
 // ------------------------------------------------------------- many tokens: by expert ---
 // With many tokens a step the (token, expert) pairs are dealt to their experts first: every
-// expert's pairs fill tiles of 32 rows (the last one padded), so that a tile's rows share the
+// expert's pairs fill tiles of 64 rows (the last one padded), so that a tile's rows share the
 // expert's matrices and the products run on the matrix cores.  A pair's row is computed from
 // the pair alone, k ascending, whatever tile and place it lands in: the result does not depend
 // on what else the step holds, nor on the order the pairs were dealt in.
 //
-// tff_experts_sort:     tile_expert[tile], tile_rows[tile * 32 + i] = pair (token * top + k) or -1,
-//                       num_tiles[0]; one block.  At most pairs / 32 + E tiles.
+// tff_experts_sort:     tile_expert[tile], tile_rows[tile * 64 + i] = pair (token * top + k) or -1,
+//                       num_tiles[0]; one block.  At most pairs / 64 + E tiles.
 // tff_experts_gate_up_tiles / tff_experts_down_tiles: the two products per tile.  The down
 //                       product writes out[k][t][:] = wts[t][k] * Wd y: `top` planes that the
 //                       norm after the feed-forward adds up in the order of k.
-#define EXT_ROWS 32
+#define EXT_ROWS 64
 
 __global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __restrict__ idx, int pairs, int E,
                                                             int max_tiles, int32_t* __restrict__ tile_expert,
@@ -270,131 +270,133 @@ __device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
     return x.v;
 }
 
-// Block: one tile of 32 pairs x 128 outputs, four waves of 32 outputs each (gate and up both).
-// C[f][pair] += W[f][k] h[pair][k]: lane (pair = lane & 15, kg = lane >> 4) ends up with outputs
-// f = kg * 4 .. + 3 of its pair.
-__global__ __launch_bounds__(256) void experts_gate_up_tiles_kernel(
-    const bf16_t* __restrict__ h, int h_row, const bf16_t* __restrict__ Wg, const bf16_t* __restrict__ Wu,
-    const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
-    const int32_t* __restrict__ num_tiles, int top, int width, int ff, float limit, float act_alpha,
-    bf16_t* __restrict__ y) {
-    const int tile = blockIdx.x;
-    if (tile >= num_tiles[0]) return;
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, kg = lane >> 4;
-    const int e = tile_expert[tile];
-    const int f0 = blockIdx.y * 128 + wv * 32;
-    if (f0 >= ff) return;       // (a whole wave)
-    int pair[2];
-    const bf16_t* hp[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        pair[i] = tile_rows[tile * EXT_ROWS + i * 16 + r];
-        hp[i] = h + (size_t)(max(pair[i], 0) / top) * h_row + kg * 8;
-    }
-    const bf16_t *gp[2], *up[2];
-    bool fok[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int f = f0 + j * 16 + r;
-        fok[j] = f < ff;
-        gp[j] = Wg + ((size_t)e * ff + min(f, ff - 1)) * width + kg * 8;
-        up[j] = Wu + ((size_t)e * ff + min(f, ff - 1)) * width + kg * 8;
-    }
-    ex_floatx4 ag[2][2], au[2][2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int i = 0; i < 2; ++i) ag[j][i] = au[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < width; k0 += 32) {
-        const bool kok = k0 + kg * 8 < width;
-        ex_bf16x8 b[2], g[2], u[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) b[i] = ex_load8(hp[i] + k0, kok && pair[i] >= 0);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            g[j] = ex_load8(gp[j] + k0, kok && fok[j]);
-            u[j] = ex_load8(up[j] + k0, kok && fok[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                ag[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g[j], b[i], ag[j][i], 0, 0, 0);
-                au[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[j], b[i], au[j][i], 0, 0, 0);
-            }
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        if (pair[i] < 0) continue;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int f = f0 + j * 16 + kg * 4 + c;
-                if (f >= ff) continue;
-                const float gv = fminf(ag[j][i][c], limit);
-                const float uv = fminf(fmaxf(au[j][i][c], -limit), limit);
-                y[(size_t)pair[i] * ff + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
-            }
-    }
-}
+// One kernel for both products.  Block: one tile of 64 pairs x 128 weight rows, four waves as 2 x 2,
+// each 32 pairs x 64 weight rows (eight accumulators).  GATE_UP: the 128 weight rows are 64 outputs
+// of the gate and the same 64 of the up projection, and a wave holds both for its outputs; else 128
+// outputs of the down projection.  K goes in steps of 64: the block's operands of a step (4 + 8
+// fragments of 16 rows x 32 k, twice) travel global -> registers while the step before is computed
+// from LDS, then registers -> LDS; a fragment lies in LDS as a wave reads it, lane l's eight
+// elements at l * 16 bytes.  C[w][pair] += W[w][k] a[pair][k]: lane (pair = lane & 15, kg = lane >> 4)
+// ends up with weight rows kg * 4 .. + 3 of its pair.  k ascends for every pair alike, whatever tile
+// and place the pair was dealt to.
+#define EXT_FRAGS 12          // fragments of a k-step of 32: 4 of the pairs' rows, 8 of the weight's
+#define EXT_KSTEP 64
 
-// Block: one tile of 32 pairs x 256 outputs of the width, four waves of 64 outputs each.
-__global__ __launch_bounds__(256) void experts_down_tiles_kernel(
-    const bf16_t* __restrict__ y, const bf16_t* __restrict__ Wd, const int32_t* __restrict__ tile_expert,
-    const int32_t* __restrict__ tile_rows, const int32_t* __restrict__ num_tiles, const float* __restrict__ wts,
-    int T, int top, int width, int ff, float* __restrict__ out) {
-    const int tile = blockIdx.x;
+template <bool GATE_UP>
+__global__ __launch_bounds__(256) void experts_tiles_kernel(
+    const bf16_t* __restrict__ a_rows, int a_row, const bf16_t* __restrict__ W0, const bf16_t* __restrict__ W1,
+    const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
+    const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
+    float limit, float act_alpha, bf16_t* __restrict__ y, float* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * EXT_FRAGS * 512];
+    const int tile = blockIdx.y;
     if (tile >= num_tiles[0]) return;
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, kg = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, r = lane & 15, kg = lane >> 4;
+    const int wm = wv & 1, wn = wv >> 1;
     const int e = tile_expert[tile];
-    const int n0 = blockIdx.y * 256 + wv * 64;
-    if (n0 >= width) return;
-    int pair[2];
-    const bf16_t* yp[2];
+    const int c0 = blockIdx.x * (GATE_UP ? 64 : 128);        // first output of the block
+    // what this thread copies each step: six 16-byte units, unit i of fragment fs = i * 4 + wv
+    const bf16_t* src[6];
+    bool ok[6];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        pair[i] = tile_rows[tile * EXT_ROWS + i * 16 + r];
-        yp[i] = y + (size_t)max(pair[i], 0) * ff + kg * 8;
+    for (int i = 0; i < 6; ++i) {
+        const int fs = i * 4 + wv, sub = fs / EXT_FRAGS, frag = fs - sub * EXT_FRAGS;
+        if (frag < 4) {
+            const int pair = tile_rows[tile * EXT_ROWS + frag * 16 + r];
+            ok[i] = pair >= 0;
+            const int row = GATE_UP ? max(pair, 0) / top : max(pair, 0);
+            src[i] = a_rows + (size_t)row * a_row + sub * 32 + kg * 8;
+        } else {
+            const int c = frag - 4;
+            int n;
+            const bf16_t* Wm = W0;
+            if (GATE_UP) {
+                n = c0 + (c & 3) * 16 + r;
+                if (c >= 4) Wm = W1;
+            } else {
+                n = c0 + c * 16 + r;
+            }
+            ok[i] = n < N;
+            src[i] = Wm + ((size_t)e * N + min(n, N - 1)) * K + sub * 32 + kg * 8;
+        }
     }
-    const bf16_t* wp[4];
-    bool nok[4];
+    auto fetch = [&](int k0, uint4 (&regs)[6]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int n = n0 + j * 16 + r;
-        nok[j] = n < width;
-        wp[j] = Wd + ((size_t)e * width + min(n, width - 1)) * ff + kg * 8;
-    }
+        for (int i = 0; i < 6; ++i) {
+            const int sub = (i * 4 + wv) / EXT_FRAGS;
+            const bool in = ok[i] && k0 + sub * 32 + kg * 8 < K;
+            regs[i] = in ? *reinterpret_cast<const uint4*>(src[i] + k0) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stash = [&](const uint4 (&regs)[6]) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+            *reinterpret_cast<uint4*>(lds + (size_t)(i * 4 + wv) * 512 + lane * 8) = regs[i];
+    };
     ex_floatx4 acc[4][2];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 2; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < ff; k0 += 32) {
-        const bool kok = k0 + kg * 8 < ff;
-        ex_bf16x8 a[4], b[2];
+    // the wave's weight fragments: gate and up of its 32 outputs, or its 64 outputs of the down projection
+    int wf[4];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) b[i] = ex_load8(yp[i] + k0, kok && pair[i] >= 0);
+    for (int j = 0; j < 4; ++j) wf[j] = GATE_UP ? (j < 2 ? wn * 2 + j : 4 + wn * 2 + (j - 2)) : wn * 4 + j;
+    uint4 regs[6];
+    fetch(0, regs);
+    for (int k0 = 0; k0 < K; k0 += EXT_KSTEP) {
+        __syncthreads();            // the step before is read
+        stash(regs);
+        __syncthreads();
+        if (k0 + EXT_KSTEP < K) fetch(k0 + EXT_KSTEP, regs);      // travels while this step is computed
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = ex_load8(wp[j] + k0, kok && nok[j]);
+        for (int sub = 0; sub < 2; ++sub) {
+            ex_bf16x8 av[2], wvv[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < 2; ++i)
+                av[i] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * EXT_FRAGS + wm * 2 + i) * 512 + lane * 8);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
+            for (int j = 0; j < 4; ++j)
+                wvv[j] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * EXT_FRAGS + 4 + wf[j]) * 512 + lane * 8);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wvv[j], av[i], acc[j][i], 0, 0, 0);
+        }
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        if (pair[i] < 0) continue;
-        const int t = pair[i] / top, k = pair[i] - t * top;
-        const float w = wts[pair[i]];
-        float* o = out + ((size_t)k * T + t) * width;
+        const int pair = tile_rows[tile * EXT_ROWS + wm * 32 + i * 16 + r];
+        if (GATE_UP) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 2; ++j) {
+                const float g4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+                const float u4[4] = {acc[2 + j][i][0], acc[2 + j][i][1], acc[2 + j][i][2], acc[2 + j][i][3]};
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int n = n0 + j * 16 + kg * 4 + c;
-                if (n < width) o[n] = w * acc[j][i][c];
+                for (int c = 0; c < 4; ++c) {
+                    const int f = c0 + (wn * 2 + j) * 16 + kg * 4 + c;
+                    if (pair >= 0 && f < N) {
+                        const float gv = fminf(g4[c], limit);
+                        const float uv = fminf(fmaxf(u4[c], -limit), limit);
+                        y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
+                    }
+                }
             }
+        } else {
+            const int p = max(pair, 0), t = p / top, k = p - t * top;
+            const float w = wts[p];
+            float* o = out + ((size_t)k * T + t) * N;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float v4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int n = c0 + (wn * 4 + j) * 16 + kg * 4 + c;
+                    if (pair >= 0 && n < N) o[n] = w * v4[c];
+                }
+            }
+        }
     }
 }
 
@@ -402,8 +404,8 @@ TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row) {
     return width % 8 == 0 && ff % 8 == 0 && h_row % 8 == 0;
 }
 
-// h [T, width] bfloat16; workspace: tile_expert [max_tiles], tile_rows [max_tiles * 32], num_tiles [1] (int32),
-// y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 32 + E.
+// h [T, width] bfloat16; workspace: tile_expert [max_tiles], tile_rows [max_tiles * 64], num_tiles [1] (int32),
+// y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 64 + E.
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
                                  float limit, float act_alpha, int32_t* tile_expert, int32_t* tile_rows,
@@ -416,19 +418,20 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
                 "multiples of 8", width, ff, h_row);
     TFF_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0 &&
                 ((uintptr_t)Wd % 16) == 0 && ((uintptr_t)y % 16) == 0, "experts_by_tiles: operands must be 16-byte aligned");
-    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles >= (long)T * top / EXT_ROWS + E,
+    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles <= 65535 && max_tiles >= (long)T * top / EXT_ROWS + E,
                 "experts_by_tiles: %d tiles do not hold %d x %d pairs of %d experts", max_tiles, T, top, E);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, max_tiles, tile_expert, tile_rows, num_tiles);
     int rc = tff_check_launch("experts_sort");
     if (rc) return rc;
-    experts_gate_up_tiles_kernel<<<dim3(max_tiles, (ff + 127) / 128), 256, 0, s>>>(
-        (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows, num_tiles, top, width, ff,
-        limit, act_alpha, (bf16_t*)y);
+    experts_tiles_kernel<true><<<dim3((ff + 63) / 64, max_tiles), 256, 0, s>>>(
+        (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows, num_tiles, wts, T, top,
+        width, ff, limit, act_alpha, (bf16_t*)y, nullptr);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
-    experts_down_tiles_kernel<<<dim3(max_tiles, (width + 255) / 256), 256, 0, s>>>(
-        (const bf16_t*)y, (const bf16_t*)Wd, tile_expert, tile_rows, num_tiles, wts, T, top, width, ff, out);
+    experts_tiles_kernel<false><<<dim3((width + 127) / 128, max_tiles), 256, 0, s>>>(
+        (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts, T, top, ff, width,
+        limit, act_alpha, nullptr, out);
     return tff_check_launch("experts_down_tiles");
 }
