@@ -185,12 +185,32 @@ __global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_
     out[i] = from_f32<T>(y);
 }
 
+// bfloat16, eight elements (16 bytes) a thread
+__global__ void gelu_bf16x8_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out, int64_t n8, int tanh_form) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    union { uint4 u; bf16_t h[8]; } a, b;
+    a.u = reinterpret_cast<const uint4*>(x)[i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float z = (float)a.h[j];
+        const float yv = tanh_form ? 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)))
+                                   : 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+        b.h[j] = (bf16_t)yv;
+    }
+    reinterpret_cast<uint4*>(out)[i] = b.u;
+}
+
 TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dtype, tff_stream_t stream) {
     TFF_REQUIRE(x && out, "gelu: null pointer");
     TFF_REQUIRE(n >= 0, "gelu: negative size");
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == TFF_BF16 && n % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        gelu_bf16x8_kernel<<<(unsigned)((n / 8 + 255) / 256), 256, 0, s>>>((const bf16_t*)x, (bf16_t*)out, n / 8, tanh_form);
+        return tff_check_launch("gelu");
+    }
     if (dtype == TFF_F32)
         gelu_kernel<float><<<blocks, 256, 0, s>>>((const float*)x, (float*)out, n, tanh_form);
     else if (dtype == TFF_BF16)

@@ -11,7 +11,9 @@
 // The two expert kernels give every (token, expert) pair waves of its own that stream the
 // expert's rows once: what a step of few tokens is bound by.  Each output element is one
 // wave's dot product in a fixed order of k, so a token's result does not depend on what else
-// the step holds.  Expert weights lie [experts, out, in], row-major.
+// the step holds.  Expert weights lie [experts, out, in], row-major, rows ldw elements apart (ldw >= in:
+// rows a power of two of bytes apart all come through one memory channel, so the loader puts a
+// little room behind each).
 #include "common.h"
 #include "tffinfer_kernels.h"
 
@@ -130,20 +132,21 @@ TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const floa
 template <typename T>
 __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
     const T* __restrict__ h, int h_row, const T* __restrict__ Wg, const T* __restrict__ Wu,
-    const int32_t* __restrict__ idx, int top, int width, int ff, float limit, float act_alpha, T* __restrict__ y) {
+    const int32_t* __restrict__ idx, int top, int width, int ff, int ldw, float limit, float act_alpha,
+    T* __restrict__ y) {
     const int pair = blockIdx.x;                  // token * top + k
     const int t = pair / top;
     const int e = idx[pair];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const T* hr = h + (size_t)t * h_row;
-    const T* wg = Wg + (size_t)e * ff * width;
-    const T* wu = Wu + (size_t)e * ff * width;
-    const bool vec = sizeof(T) == 2 && width % 8 == 0 && h_row % 8 == 0 && ((uintptr_t)h % 16) == 0 &&
+    const T* wg = Wg + (size_t)e * ff * ldw;
+    const T* wu = Wu + (size_t)e * ff * ldw;
+    const bool vec = sizeof(T) == 2 && width % 8 == 0 && ldw % 8 == 0 && h_row % 8 == 0 && ((uintptr_t)h % 16) == 0 &&
                      ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0;
     const int f0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
     for (int f = f0; f < min(ff, f0 + EX_PER_WAVE); ++f) {
-        float g = row_dot<T>(hr, wg + (size_t)f * width, width, lane, vec);
-        float u = row_dot<T>(hr, wu + (size_t)f * width, width, lane, vec);
+        float g = row_dot<T>(hr, wg + (size_t)f * ldw, width, lane, vec);
+        float u = row_dot<T>(hr, wu + (size_t)f * ldw, width, lane, vec);
         if (lane == 0) {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
@@ -156,16 +159,16 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
 template <typename T>
 __global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
     const T* __restrict__ y, const T* __restrict__ Wd, const int32_t* __restrict__ idx, const float* __restrict__ wts,
-    int top, int width, int ff, float* __restrict__ out) {
+    int top, int width, int ff, int ldw, float* __restrict__ out) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const bool vec = sizeof(T) == 2 && ff % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)Wd % 16) == 0;
+    const bool vec = sizeof(T) == 2 && ff % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)Wd % 16) == 0;
     const int n0 = (blockIdx.y * EX_WAVES + wv) * EX_PER_WAVE;
     for (int n = n0; n < min(width, n0 + EX_PER_WAVE); ++n) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k) {
             const int e = idx[(size_t)t * top + k];
-            const float d = row_dot<T>(y + ((size_t)t * top + k) * ff, Wd + ((size_t)e * width + n) * ff, ff, lane, vec);
+            const float d = row_dot<T>(y + ((size_t)t * top + k) * ff, Wd + ((size_t)e * width + n) * ldw, ff, lane, vec);
             acc = fmaf(wts[(size_t)t * top + k], d, acc);
         }
         if (lane == 0) out[(size_t)t * width + n] = acc;
@@ -173,10 +176,10 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
 }
 
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, float limit, float act_alpha, void* y, int dtype,
-                                tff_stream_t stream) {
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, void* y,
+                                int dtype, tff_stream_t stream) {
     TFF_REQUIRE(h && Wg && Wu && idx && y, "experts_gate_up: null pointer");
-    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width,
+    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width && ldw >= width,
                 "experts_gate_up: bad sizes T=%d top=%d width=%d ff=%d", T, top, width, ff);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -184,10 +187,10 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
     TFF_REQUIRE(grid.y <= 65535, "experts_gate_up: too many outputs");
     if (dtype == TFF_F32)
         experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)h, h_row, (const float*)Wg, (const float*)Wu,
-                                                                    idx, top, width, ff, limit, act_alpha, (float*)y);
+                                                                    idx, top, width, ff, ldw, limit, act_alpha, (float*)y);
     else if (dtype == TFF_BF16)
         experts_gate_up_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)h, h_row, (const bf16_t*)Wg,
-                                                                     (const bf16_t*)Wu, idx, top, width, ff, limit,
+                                                                     (const bf16_t*)Wu, idx, top, width, ff, ldw, limit,
                                                                      act_alpha, (bf16_t*)y);
     else
         return tff_fail("experts_gate_up: unknown dtype %d", dtype);
@@ -195,18 +198,18 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
 }
 
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
-                             int width, int ff, float* out, int dtype, tff_stream_t stream) {
+                             int width, int ff, int ldw, float* out, int dtype, tff_stream_t stream) {
     TFF_REQUIRE(y && Wd && idx && wts && out, "experts_down: null pointer");
-    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0, "experts_down: bad sizes T=%d top=%d width=%d ff=%d",
+    TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && ldw >= ff, "experts_down: bad sizes T=%d top=%d width=%d ff=%d",
                 T, top, width, ff);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(T, (width + EX_WAVES * EX_PER_WAVE - 1) / (EX_WAVES * EX_PER_WAVE));
     TFF_REQUIRE(grid.y <= 65535, "experts_down: too many outputs");
     if (dtype == TFF_F32)
-        experts_down_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)y, (const float*)Wd, idx, wts, top, width, ff, out);
+        experts_down_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)y, (const float*)Wd, idx, wts, top, width, ff, ldw, out);
     else if (dtype == TFF_BF16)
-        experts_down_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)y, (const bf16_t*)Wd, idx, wts, top, width, ff, out);
+        experts_down_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)y, (const bf16_t*)Wd, idx, wts, top, width, ff, ldw, out);
     else
         return tff_fail("experts_down: unknown dtype %d", dtype);
     return tff_check_launch("experts_down");
@@ -270,16 +273,17 @@ __device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
     return x.v;
 }
 
-// One kernel for both products.  Block: one tile of 64 pairs x 128 weight rows, four waves as 2 x 2,
-// each 32 pairs x 64 weight rows (eight accumulators).  GATE_UP: the 128 weight rows are 64 outputs
-// of the gate and the same 64 of the up projection, and a wave holds both for its outputs; else 128
-// outputs of the down projection.  K goes in steps of 64: the block's operands of a step (4 + 8
-// fragments of 16 rows x 32 k, twice) travel global -> registers while the step before is computed
-// from LDS, then registers -> LDS; a fragment lies in LDS as a wave reads it, lane l's eight
-// elements at l * 16 bytes.  C[w][pair] += W[w][k] a[pair][k]: lane (pair = lane & 15, kg = lane >> 4)
-// ends up with weight rows kg * 4 .. + 3 of its pair.  k ascends for every pair alike, whatever tile
-// and place the pair was dealt to.
-#define EXT_FRAGS 12          // fragments of a k-step of 32: 4 of the pairs' rows, 8 of the weight's
+// One kernel for both products.  Block: one tile of 64 pairs x 128 weight rows, four waves side by
+// side, each all 64 pairs x 32 weight rows (eight accumulators).  GATE_UP: a wave's 32 weight rows
+// are 16 outputs of the gate and the same 16 of the up projection; else 32 outputs of the down
+// projection.  K goes in steps of 64.  The pairs' rows, which all four waves need, pass through LDS
+// (global -> registers while the step before is computed, then registers -> LDS; a fragment of 16
+// rows x 32 k lies there as a wave reads it, lane l's eight elements at l * 16 bytes); a wave's own
+// weight rows go straight from memory into its MFMA operands, one step ahead: LDS bandwidth is what
+// bounds a block of few waves, and the weight is two thirds of the operands.
+// C[w][pair] += W[w][k] a[pair][k]: lane (pair = lane & 15, kg = lane >> 4) ends up with weight rows
+// kg * 4 .. + 3 of its pair.  k ascends for every pair alike, whatever tile and place the pair was
+// dealt to.
 #define EXT_KSTEP 64
 
 template <bool GATE_UP>
@@ -287,100 +291,96 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const bf16_t* __restrict__ a_rows, int a_row, const bf16_t* __restrict__ W0, const bf16_t* __restrict__ W1,
     const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
     const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
-    float limit, float act_alpha, bf16_t* __restrict__ y, float* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * EXT_FRAGS * 512];
-    const int tile = blockIdx.y;
-    if (tile >= num_tiles[0]) return;
+    float limit, float act_alpha, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
+    int ldw) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * 4 * 512];      // two sub-steps of four fragments
+    // A tile of 64 pairs gives a weight element 128 flops a read: the tiles of one expert must meet
+    // their weight rows in a cache, or the products run at what memory gives.  Blocks go to the
+    // eight XCDs in turn by their number, each XCD with an L2 of its own; so block L works on
+    // column block (L / 8 / max_tiles) * 8 + L % 8 and tile L / 8 % max_tiles: one XCD sees all
+    // tiles of a column block one after the other, an expert's tiles next to each other.
+    const int L = blockIdx.x, q = L >> 3;
+    const int tile = q % max_tiles, col_block = (q / max_tiles) * 8 + (L & 7);
+    if (tile >= num_tiles[0] || col_block >= col_blocks) return;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, r = lane & 15, kg = lane >> 4;
-    const int wm = wv & 1, wn = wv >> 1;
     const int e = tile_expert[tile];
-    const int c0 = blockIdx.x * (GATE_UP ? 64 : 128);        // first output of the block
-    // what this thread copies each step: six 16-byte units, unit i of fragment fs = i * 4 + wv
-    const bf16_t* src[6];
-    bool ok[6];
-#pragma unroll
-    for (int i = 0; i < 6; ++i) {
-        const int fs = i * 4 + wv, sub = fs / EXT_FRAGS, frag = fs - sub * EXT_FRAGS;
-        if (frag < 4) {
-            const int pair = tile_rows[tile * EXT_ROWS + frag * 16 + r];
-            ok[i] = pair >= 0;
-            const int row = GATE_UP ? max(pair, 0) / top : max(pair, 0);
-            src[i] = a_rows + (size_t)row * a_row + sub * 32 + kg * 8;
-        } else {
-            const int c = frag - 4;
-            int n;
-            const bf16_t* Wm = W0;
-            if (GATE_UP) {
-                n = c0 + (c & 3) * 16 + r;
-                if (c >= 4) Wm = W1;
-            } else {
-                n = c0 + c * 16 + r;
-            }
-            ok[i] = n < N;
-            src[i] = Wm + ((size_t)e * N + min(n, N - 1)) * K + sub * 32 + kg * 8;
-        }
-    }
-    auto fetch = [&](int k0, uint4 (&regs)[6]) {
-#pragma unroll
-        for (int i = 0; i < 6; ++i) {
-            const int sub = (i * 4 + wv) / EXT_FRAGS;
-            const bool in = ok[i] && k0 + sub * 32 + kg * 8 < K;
-            regs[i] = in ? *reinterpret_cast<const uint4*>(src[i] + k0) : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto stash = [&](const uint4 (&regs)[6]) {
-#pragma unroll
-        for (int i = 0; i < 6; ++i)
-            *reinterpret_cast<uint4*>(lds + (size_t)(i * 4 + wv) * 512 + lane * 8) = regs[i];
-    };
-    ex_floatx4 acc[4][2];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < 2; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
-    // the wave's weight fragments: gate and up of its 32 outputs, or its 64 outputs of the down projection
-    int wf[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) wf[j] = GATE_UP ? (j < 2 ? wn * 2 + j : 4 + wn * 2 + (j - 2)) : wn * 4 + j;
-    uint4 regs[6];
-    fetch(0, regs);
-    for (int k0 = 0; k0 < K; k0 += EXT_KSTEP) {
-        __syncthreads();            // the step before is read
-        stash(regs);
-        __syncthreads();
-        if (k0 + EXT_KSTEP < K) fetch(k0 + EXT_KSTEP, regs);      // travels while this step is computed
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            ex_bf16x8 av[2], wvv[4];
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                av[i] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * EXT_FRAGS + wm * 2 + i) * 512 + lane * 8);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                wvv[j] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * EXT_FRAGS + 4 + wf[j]) * 512 + lane * 8);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 2; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wvv[j], av[i], acc[j][i], 0, 0, 0);
-        }
-    }
+    const int c0 = col_block * (GATE_UP ? 64 : 128) + wv * (GATE_UP ? 16 : 32);     // the wave's first output
+    // the pairs' rows: eight fragments a step (four of 16 pairs, two sub-steps of 32 k), two a wave
+    const bf16_t* asrc[2];
+    bool aok[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int pair = tile_rows[tile * EXT_ROWS + wm * 32 + i * 16 + r];
+        const int fs = i * 4 + wv, sub = fs >> 2, frag = fs & 3;
+        const int pair = tile_rows[tile * EXT_ROWS + frag * 16 + r];
+        aok[i] = pair >= 0;
+        asrc[i] = a_rows + (size_t)(GATE_UP ? max(pair, 0) / top : max(pair, 0)) * a_row + sub * 32 + kg * 8;
+    }
+    // the wave's weight rows: two fragments
+    const bf16_t* wsrc[2];
+    bool wok[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = GATE_UP ? c0 + r : c0 + j * 16 + r;
+        wok[j] = n < N;
+        wsrc[j] = ((GATE_UP && j == 1) ? W1 : W0) + ((size_t)e * N + min(n, N - 1)) * ldw + kg * 8;
+    }
+    ex_floatx4 acc[2][4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
+    uint4 areg[2];
+    ex_bf16x8 wreg[2][2];        // [sub][fragment] of the step that is fetched
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int sub = (i * 4 + wv) >> 2;
+            const bool in = aok[i] && k0 + sub * 32 + kg * 8 < K;
+            areg[i] = in ? *reinterpret_cast<const uint4*>(asrc[i] + k0) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) wreg[sub][j] = ex_load8(wsrc[j] + k0 + sub * 32, wok[j] && k0 + sub * 32 + kg * 8 < K);
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += EXT_KSTEP) {
+        __syncthreads();            // the step before is read
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(i * 4 + wv) * 512 + lane * 8) = areg[i];
+        ex_bf16x8 wnow[2][2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) wnow[sub][j] = wreg[sub][j];
+        __syncthreads();
+        if (k0 + EXT_KSTEP < K) fetch(k0 + EXT_KSTEP);      // travels while this step is computed
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            ex_bf16x8 av[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                av[i] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * 4 + i) * 512 + lane * 8);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wnow[sub][j], av[i], acc[j][i], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pair = tile_rows[tile * EXT_ROWS + i * 16 + r];
         if (GATE_UP) {
+            const float g4[4] = {acc[0][i][0], acc[0][i][1], acc[0][i][2], acc[0][i][3]};
+            const float u4[4] = {acc[1][i][0], acc[1][i][1], acc[1][i][2], acc[1][i][3]};
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const float g4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
-                const float u4[4] = {acc[2 + j][i][0], acc[2 + j][i][1], acc[2 + j][i][2], acc[2 + j][i][3]};
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int f = c0 + (wn * 2 + j) * 16 + kg * 4 + c;
-                    if (pair >= 0 && f < N) {
-                        const float gv = fminf(g4[c], limit);
-                        const float uv = fminf(fmaxf(u4[c], -limit), limit);
-                        y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
-                    }
+            for (int c = 0; c < 4; ++c) {
+                const int f = c0 + kg * 4 + c;
+                if (pair >= 0 && f < N) {
+                    const float gv = fminf(g4[c], limit);
+                    const float uv = fminf(fmaxf(u4[c], -limit), limit);
+                    y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
                 }
             }
         } else {
@@ -388,11 +388,11 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
             const float w = wts[p];
             float* o = out + ((size_t)k * T + t) * N;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < 2; ++j) {
                 const float v4[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const int n = c0 + (wn * 4 + j) * 16 + kg * 4 + c;
+                    const int n = c0 + j * 16 + kg * 4 + c;
                     if (pair >= 0 && n < N) o[n] = w * v4[c];
                 }
             }
@@ -408,30 +408,33 @@ TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row) {
 // y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 64 + E.
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
-                                 float limit, float act_alpha, int32_t* tile_expert, int32_t* tile_rows,
-                                 int32_t* num_tiles, int max_tiles, void* y, float* out, tff_stream_t stream) {
+                                 int ldw_in, int ldw_down, float limit, float act_alpha, int32_t* tile_expert,
+                                 int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
+                                 tff_stream_t stream) {
     TFF_REQUIRE(h && Wg && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
                 "experts_by_tiles: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= RT_MAX_E && width > 0 && ff > 0 && h_row >= width,
                 "experts_by_tiles: bad sizes T=%d top=%d E=%d width=%d ff=%d", T, top, E, width, ff);
-    TFF_REQUIRE(tff_experts_tiles_supported(width, ff, h_row), "experts_by_tiles: width %d, ff %d and rows of %d must be "
-                "multiples of 8", width, ff, h_row);
+    TFF_REQUIRE(tff_experts_tiles_supported(width, ff, h_row) && ldw_in % 8 == 0 && ldw_down % 8 == 0 && ldw_in >= width &&
+                ldw_down >= ff, "experts_by_tiles: width %d, ff %d, rows of %d and the weights' rows of %d and %d must be "
+                "multiples of 8", width, ff, h_row, ldw_in, ldw_down);
     TFF_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0 &&
                 ((uintptr_t)Wd % 16) == 0 && ((uintptr_t)y % 16) == 0, "experts_by_tiles: operands must be 16-byte aligned");
-    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles <= 65535 && max_tiles >= (long)T * top / EXT_ROWS + E,
+    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles <= (1 << 20) && max_tiles >= (long)T * top / EXT_ROWS + E,
                 "experts_by_tiles: %d tiles do not hold %d x %d pairs of %d experts", max_tiles, T, top, E);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, max_tiles, tile_expert, tile_rows, num_tiles);
     int rc = tff_check_launch("experts_sort");
     if (rc) return rc;
-    experts_tiles_kernel<true><<<dim3((ff + 63) / 64, max_tiles), 256, 0, s>>>(
+    const int cb_up = (ff + 63) / 64, cb_down = (width + 127) / 128;
+    experts_tiles_kernel<true><<<(cb_up + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(
         (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows, num_tiles, wts, T, top,
-        width, ff, limit, act_alpha, (bf16_t*)y, nullptr);
+        width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
-    experts_tiles_kernel<false><<<dim3((width + 127) / 128, max_tiles), 256, 0, s>>>(
+    experts_tiles_kernel<false><<<(cb_down + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(
         (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts, T, top, ff, width,
-        limit, act_alpha, nullptr, out);
+        limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
     return tff_check_launch("experts_down_tiles");
 }

@@ -260,13 +260,13 @@ TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dty
 TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
                            int width, int E, int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
 // y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + 1), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
-// e = idx[t, k]; Wg, Wu [E, ff, width].
+// e = idx[t, k]; Wg, Wu [E, ff, width], rows ldw elements apart.
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, float limit, float act_alpha, void* y, int dtype,
-                                tff_stream_t stream);
-// out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff]; out float32.
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, void* y,
+                                int dtype, tff_stream_t stream);
+// out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff], rows ldw elements apart; out float32.
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
-                             int width, int ff, float* out, int dtype, tff_stream_t stream);
+                             int width, int ff, int ldw, float* out, int dtype, tff_stream_t stream);
 
 // The same for steps of many tokens (bfloat16; width, ff and h_row multiples of 8): the (token, expert) pairs
 // are dealt to their experts in tiles of 64 rows and the two products run on the matrix cores.  out is
@@ -276,8 +276,9 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row);
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
-                                 float limit, float act_alpha, int32_t* tile_expert, int32_t* tile_rows,
-                                 int32_t* num_tiles, int max_tiles, void* y, float* out, tff_stream_t stream);
+                                 int ldw_in, int ldw_down, float limit, float act_alpha, int32_t* tile_expert,
+                                 int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
+                                 tff_stream_t stream);
 
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

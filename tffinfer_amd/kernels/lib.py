@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 
 
 class KernelLibraryError(RuntimeError):
@@ -51,10 +51,10 @@ _SIGNATURES = {
     "tff_scale_add_rmsnorm": [_P, _P, _I, _Z, _F, _P, _F, _P, _I, _I, _I, _P],
     "tff_gelu": [_P, _P, c_int64, _I, _I, _P],
     "tff_route_topk": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P],
-    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _I, _P],
+    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P, _I, _P],
     "tff_experts_tiles_supported": [_I, _I, _I],
-    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _P, _P, _I, _P, _P, _P],
-    "tff_experts_down": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _P],
+    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _P, _P, _I, _P, _P, _P],
+    "tff_experts_down": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],
     "tff_argmax_workspace_bytes": [_I, _I],

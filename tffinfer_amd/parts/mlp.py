@@ -149,7 +149,8 @@ class RoutedExperts(FeedForward):
         E = self.num_experts
 
         def stack(which):
-            return torch.stack([weights[f"e{e}.{which}"].to(dtype) for e in range(E)], 0).contiguous().to(device)
+            from ..kernels.ops import pad_expert_rows
+            return pad_expert_rows(torch.stack([weights[f"e{e}.{which}"].to(dtype) for e in range(E)], 0)).to(device)
 
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         # The router's logits are float32 sums.  A router stored in bfloat16 multiplies exactly with
