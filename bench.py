@@ -81,6 +81,12 @@ def design_points(args):
             if args.design_only and label != args.design_only and not label.startswith(args.design_only):
                 continue
             model = build_model(dict(cfg), args.seed)
+            for block in model.blocks:
+                # (random corrections of the scores' own size would send every token to the same few
+                # experts; without them the random router spreads the tokens over all of them)
+                corr = getattr(block.feed_forward, "correction", None)
+                if corr is not None:
+                    corr.zero_()
             vocab = model.config.vocab_size
             total = steps + warmup + M.decode_slack(batch, context) + 16
             opt = EngineOptions(dtype="bfloat16", page_size=args.page_size,
