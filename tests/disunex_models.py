@@ -68,10 +68,16 @@ DX_S = {"architecture": "Disunex", "width": 60, "vocab": 101, "postln_alpha": 0.
     layer(mixer(3, 10, 6, 14, 20, 0.3, window=9), dense(50), weights_of=0),
     layer(mixer(2, 6, 2, 5, 11, 0.4), moe(4, 2, 12, 2.0)),
 ]}
-DISUNEX_CONFIGS = {"dxP": (DX_P, 3), "dxQ": (DX_Q, 5), "dxR": (DX_R, 7), "dxS": (DX_S, 9)}
-DISUNEX_PAGE = {"dxP": 16, "dxQ": 8, "dxR": 16, "dxS": 32}
+# a key of 288 elements, beyond what the matrix-core attention takes (the general kernel in both types),
+# and a mixture in which every expert is chosen
+DX_T = {"architecture": "Disunex", "width": 48, "vocab": 90, "postln_alpha": 1.5, "norm": {"eps": 1e-5}, "layers": [
+    layer(mixer(2, 8, 8, 16, 280, 0.3, window=10), moe(2, 2, 16, 1.0), weights_of=1),
+    layer(mixer(2, 8, 8, 16, 280, 0.3, window=10), moe(2, 2, 16, 1.0)),
+]}
+DISUNEX_CONFIGS = {"dxP": (DX_P, 3), "dxQ": (DX_Q, 5), "dxR": (DX_R, 7), "dxS": (DX_S, 9), "dxT": (DX_T, 13)}
+DISUNEX_PAGE = {"dxP": 16, "dxQ": 8, "dxR": 16, "dxS": 32, "dxT": 16}
 DISUNEX_LENGTHS = {"dxP": [1, 2, 11, 12, 13, 40, 61], "dxQ": [3, 36, 37, 38, 75, 130], "dxR": [5, 33, 34, 70],
-                   "dxS": [2, 9, 10, 33, 80]}
+                   "dxS": [2, 9, 10, 33, 80], "dxT": [1, 10, 11, 50]}
 
 #: factors on the drawn weights by the tensor's last name
 SHARP = {"q": 10.0, "uk": 10.0, "dkv": 6.0, "g": 10.0, "uv": 5.0, "o": 5.0, "up": 6.0, "down": 6.0, "gate": 10.0,

@@ -28,6 +28,15 @@ def test_layers_that_borrow_tensors_are_calls_of_their_owner_with_a_cache_of_the
     assert specs[0].num_kv_heads == 1 and specs[0].window == 12 and specs[3].window == 0
 
 
+def test_a_layer_may_borrow_from_a_later_one_and_a_large_key_is_padded_to_a_multiple_of_8():
+    from disunex_models import DX_T
+    cfg = config_from_dict(copy.deepcopy(DX_T))
+    assert cfg.owners() == [1] and cfg.layer_schedule() == [LayerCall(0, 0), LayerCall(0, 1)]
+    model = build_model_skeleton(cfg)
+    assert sorted(n for n in model.expected_tensors() if n.endswith("norm1")) == ["l1.norm1"]
+    assert model.blocks[0].mixer.cache_spec().head_dim == 288
+
+
 def test_every_size_comes_from_the_file():
     cfg = config_from_dict(copy.deepcopy(DX_R))
     m = build_model_skeleton(cfg).blocks[0].mixer

@@ -15,7 +15,7 @@ from helpers import note_error, oracle_logits, random_tokens, read_config, rel_e
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-NAMES = ["dxP", "dxQ", "dxR", "dxS"]
+NAMES = ["dxP", "dxQ", "dxR", "dxS", "dxT"]
 
 
 def _ops():
