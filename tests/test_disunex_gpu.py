@@ -87,7 +87,7 @@ def test_router_choice_goes_by_the_corrected_scores_and_weights_by_the_plain_one
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T", [19, 150])
+@pytest.mark.parametrize("T", [19, 150, 700])          # (700: tiles of 128 pairs where the experts are few)
 @pytest.mark.parametrize("E,top,width,ff,limit", [(5, 2, 64, 40, 0.7), (3, 1, 100, 24, 1.5), (6, 3, 72, 17, 0.5),
                                                   (40, 4, 264, 136, 0.8)])
 def test_experts(dtype, E, top, width, ff, limit, T):

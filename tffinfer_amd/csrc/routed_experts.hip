@@ -217,7 +217,7 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 
 // ------------------------------------------------------------- many tokens: by expert ---
 // With many tokens a step the (token, expert) pairs are dealt to their experts first: every
-// expert's pairs fill tiles of 64 rows (the last one padded), so that a tile's rows share the
+// expert's pairs fill tiles of 64 rows (128 where the experts have a few hundred pairs each) (the last one padded), so that a tile's rows share the
 // expert's matrices and the products run on the matrix cores.  A pair's row is computed from
 // the pair alone, k ascending, whatever tile and place it lands in: the result does not depend
 // on what else the step holds, nor on the order the pairs were dealt in.
@@ -227,10 +227,9 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 // tff_experts_gate_up_tiles / tff_experts_down_tiles: the two products per tile.  The down
 //                       product writes out[k][t][:] = wts[t][k] * Wd y: `top` planes that the
 //                       norm after the feed-forward adds up in the order of k.
-#define EXT_ROWS 64
 
 __global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __restrict__ idx, int pairs, int E,
-                                                            int max_tiles, int32_t* __restrict__ tile_expert,
+                                                            int rows, int32_t* __restrict__ tile_expert,
                                                             int32_t* __restrict__ tile_rows,
                                                             int32_t* __restrict__ num_tiles) {
     __shared__ int count[RT_MAX_E];
@@ -244,7 +243,7 @@ __global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __res
         int t = 0;
         for (int e = 0; e < E; ++e) {
             first[e] = t;
-            t += (count[e] + EXT_ROWS - 1) / EXT_ROWS;
+            t += (count[e] + rows - 1) / rows;
         }
         first[E] = t;
         num_tiles[0] = t;
@@ -255,12 +254,12 @@ __global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __res
         for (int t = first[e]; t < first[e + 1]; ++t) tile_expert[t] = e;
         count[e] = 0;
     }
-    for (int i = tid; i < tiles * EXT_ROWS; i += blockDim.x) tile_rows[i] = -1;
+    for (int i = tid; i < tiles * rows; i += blockDim.x) tile_rows[i] = -1;
     __syncthreads();
     for (int p = tid; p < pairs; p += blockDim.x) {
         const int e = idx[p];
         const int at = atomicAdd(&count[e], 1);
-        tile_rows[first[e] * EXT_ROWS + at] = p;
+        tile_rows[first[e] * rows + at] = p;
     }
 }
 
@@ -273,8 +272,8 @@ __device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
     return x.v;
 }
 
-// One kernel for both products.  Block: one tile of 64 pairs x 128 weight rows, four waves side by
-// side, each all 64 pairs x 32 weight rows (eight accumulators).  GATE_UP: a wave's 32 weight rows
+// One kernel for both products.  Block: one tile of 64 or 128 pairs x 128 weight rows, four waves side by
+// side, each all pairs x 32 weight rows (eight or sixteen accumulators).  GATE_UP: a wave's 32 weight rows
 // are 16 outputs of the gate and the same 16 of the up projection; else 32 outputs of the down
 // projection.  K goes in steps of 64.  The pairs' rows, which all four waves need, pass through LDS
 // (global -> registers while the step before is computed, then registers -> LDS; a fragment of 16
@@ -286,14 +285,15 @@ __device__ __forceinline__ ex_bf16x8 ex_load8(const bf16_t* p, bool ok) {
 // dealt to.
 #define EXT_KSTEP 64
 
-template <bool GATE_UP>
+template <bool GATE_UP, int AFR>
 __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const bf16_t* __restrict__ a_rows, int a_row, const bf16_t* __restrict__ W0, const bf16_t* __restrict__ W1,
     const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
     const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
     float limit, float act_alpha, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
     int ldw) {
-    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * 4 * 512];      // two sub-steps of four fragments
+    constexpr int ROWS = AFR * 16;       // pairs of a tile: 64, or 128 where the experts have many pairs each
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * AFR * 512];      // two sub-steps of AFR fragments
     // A tile of 64 pairs gives a weight element 128 flops a read: the tiles of one expert must meet
     // their weight rows in a cache, or the products run at what memory gives.  Blocks go to the
     // eight XCDs in turn by their number, each XCD with an L2 of its own; so block L works on
@@ -305,13 +305,14 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, r = lane & 15, kg = lane >> 4;
     const int e = tile_expert[tile];
     const int c0 = col_block * (GATE_UP ? 64 : 128) + wv * (GATE_UP ? 16 : 32);     // the wave's first output
-    // the pairs' rows: eight fragments a step (four of 16 pairs, two sub-steps of 32 k), two a wave
-    const bf16_t* asrc[2];
-    bool aok[2];
+    // the pairs' rows: 2 AFR fragments a step (AFR of 16 pairs, two sub-steps of 32 k), AFR / 2 a wave
+    constexpr int AU = AFR / 2;
+    const bf16_t* asrc[AU];
+    bool aok[AU];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int fs = i * 4 + wv, sub = fs >> 2, frag = fs & 3;
-        const int pair = tile_rows[tile * EXT_ROWS + frag * 16 + r];
+    for (int i = 0; i < AU; ++i) {
+        const int fs = i * 4 + wv, sub = fs / AFR, frag = fs % AFR;
+        const int pair = tile_rows[tile * ROWS + frag * 16 + r];
         aok[i] = pair >= 0;
         asrc[i] = a_rows + (size_t)(GATE_UP ? max(pair, 0) / top : max(pair, 0)) * a_row + sub * 32 + kg * 8;
     }
@@ -324,17 +325,17 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
         wok[j] = n < N;
         wsrc[j] = ((GATE_UP && j == 1) ? W1 : W0) + ((size_t)e * N + min(n, N - 1)) * ldw + kg * 8;
     }
-    ex_floatx4 acc[2][4];
+    ex_floatx4 acc[2][AFR];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
-    uint4 areg[2];
+        for (int i = 0; i < AFR; ++i) acc[j][i] = ex_floatx4{0.f, 0.f, 0.f, 0.f};
+    uint4 areg[AU];
     ex_bf16x8 wreg[2][2];        // [sub][fragment] of the step that is fetched
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int sub = (i * 4 + wv) >> 2;
+        for (int i = 0; i < AU; ++i) {
+            const int sub = (i * 4 + wv) / AFR;
             const bool in = aok[i] && k0 + sub * 32 + kg * 8 < K;
             areg[i] = in ? *reinterpret_cast<const uint4*>(asrc[i] + k0) : make_uint4(0, 0, 0, 0);
         }
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
     for (int k0 = 0; k0 < K; k0 += EXT_KSTEP) {
         __syncthreads();            // the step before is read
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(i * 4 + wv) * 512 + lane * 8) = areg[i];
+        for (int i = 0; i < AU; ++i) *reinterpret_cast<uint4*>(lds + (size_t)(i * 4 + wv) * 512 + lane * 8) = areg[i];
         ex_bf16x8 wnow[2][2];
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub)
@@ -357,20 +358,20 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
         if (k0 + EXT_KSTEP < K) fetch(k0 + EXT_KSTEP);      // travels while this step is computed
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
-            ex_bf16x8 av[4];
+            ex_bf16x8 av[AFR];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                av[i] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * 4 + i) * 512 + lane * 8);
+            for (int i = 0; i < AFR; ++i)
+                av[i] = *reinterpret_cast<const ex_bf16x8*>(lds + (size_t)(sub * AFR + i) * 512 + lane * 8);
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < AFR; ++i)
                     acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wnow[sub][j], av[i], acc[j][i], 0, 0, 0);
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int pair = tile_rows[tile * EXT_ROWS + i * 16 + r];
+    for (int i = 0; i < AFR; ++i) {
+        const int pair = tile_rows[tile * ROWS + i * 16 + r];
         if (GATE_UP) {
             const float g4[4] = {acc[0][i][0], acc[0][i][1], acc[0][i][2], acc[0][i][3]};
             const float u4[4] = {acc[1][i][0], acc[1][i][1], acc[1][i][2], acc[1][i][3]};
@@ -404,7 +405,7 @@ TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row) {
     return width % 8 == 0 && ff % 8 == 0 && h_row % 8 == 0;
 }
 
-// h [T, width] bfloat16; workspace: tile_expert [max_tiles], tile_rows [max_tiles * 64], num_tiles [1] (int32),
+// h [T, width] bfloat16; workspace: tile_expert [max_tiles], tile_rows [max_tiles * 128], num_tiles [1] (int32),
 // y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 64 + E.
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
@@ -420,21 +421,34 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
                 "multiples of 8", width, ff, h_row, ldw_in, ldw_down);
     TFF_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)Wg % 16) == 0 && ((uintptr_t)Wu % 16) == 0 &&
                 ((uintptr_t)Wd % 16) == 0 && ((uintptr_t)y % 16) == 0, "experts_by_tiles: operands must be 16-byte aligned");
-    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles <= (1 << 20) && max_tiles >= (long)T * top / EXT_ROWS + E,
+    TFF_REQUIRE((long)T * top < (1L << 31) && max_tiles <= (1 << 20) && max_tiles >= (long)T * top / 64 + E,
                 "experts_by_tiles: %d tiles do not hold %d x %d pairs of %d experts", max_tiles, T, top, E);
+    // tiles of 128 pairs where an expert has a few hundred on average: every weight element fetched
+    // serves twice the flops, which is what bounds these products; the padding of an expert's last
+    // tile costs more with fewer pairs
+    const bool tall = (long)T * top >= 192L * E;
+    const int rows = tall ? 128 : 64;
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, max_tiles, tile_expert, tile_rows, num_tiles);
+    experts_sort_kernel<<<1, 1024, 0, s>>>(idx, T * top, E, rows, tile_expert, tile_rows, num_tiles);
     int rc = tff_check_launch("experts_sort");
     if (rc) return rc;
     const int cb_up = (ff + 63) / 64, cb_down = (width + 127) / 128;
-    experts_tiles_kernel<true><<<(cb_up + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(
-        (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows, num_tiles, wts, T, top,
-        width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+#define EXT_LAUNCH(GU, AFRV, CB, ...) experts_tiles_kernel<GU, AFRV><<<((CB) + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(__VA_ARGS__)
+    if (tall)
+        EXT_LAUNCH(true, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+    else
+        EXT_LAUNCH(true, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
-    experts_tiles_kernel<false><<<(cb_down + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(
-        (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts, T, top, ff, width,
-        limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
+    if (tall)
+        EXT_LAUNCH(false, 8, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
+                   T, top, ff, width, limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
+    else
+        EXT_LAUNCH(false, 4, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
+                   T, top, ff, width, limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
+#undef EXT_LAUNCH
     return tff_check_launch("experts_down_tiles");
 }

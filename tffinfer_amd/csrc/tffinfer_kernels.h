@@ -269,9 +269,9 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
                              int width, int ff, int ldw, float* out, int dtype, tff_stream_t stream);
 
 // The same for steps of many tokens (bfloat16; width, ff and h_row multiples of 8): the (token, expert) pairs
-// are dealt to their experts in tiles of 64 rows and the two products run on the matrix cores.  out is
+// are dealt to their experts in tiles of 64 or 128 rows and the two products run on the matrix cores.  out is
 // float32 [top, T, width], plane k = wts[:, k] * (expert k's output): the consumer adds the planes in order.
-// Workspace: tile_expert [max_tiles], tile_rows [64 * max_tiles], num_tiles [1], y [T * top, ff] bfloat16;
+// Workspace: tile_expert [max_tiles], tile_rows [128 * max_tiles], num_tiles [1], y [T * top, ff] bfloat16;
 // max_tiles >= T * top / 64 + E.
 TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row);
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,

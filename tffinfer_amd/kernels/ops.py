@@ -1093,12 +1093,12 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
         # many tokens: the pairs dealt to their experts, the products on the matrix cores; the result
         # comes as one plane per chosen expert, for the norm that follows to add up in their order
         max_tiles = T * top // 64 + E
-        tables = torch.empty(65 * max_tiles + 1, dtype=torch.int32, device=h.device)
+        tables = torch.empty(129 * max_tiles + 1, dtype=torch.int32, device=h.device)
         out = torch.empty(top, T, width, dtype=torch.float32, device=h.device)
         _lib.check(L.tff_experts_by_tiles(
             h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
             T, top, E, width, ff, ld_in, ld_down, float(limit), float(act_alpha), tables.data_ptr(), tables[max_tiles:].data_ptr(),
-            tables[65 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
+            tables[129 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
         return out if top > 1 else out[0]
     _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), idx.data_ptr(), T, top, E,
                                      width, ff, ld_in, float(limit), float(act_alpha), y.data_ptr(), dtype_code(h.dtype),
