@@ -416,3 +416,32 @@ def test_the_command_line_with_a_configuration_file_of_this_architecture(tmp_pat
     assert tight.returncode == 0, tight.stderr[-3000:]
     assert "preemption" in tight.stderr
     assert [json.loads(ln)["output"] for ln in tight.stdout.strip().splitlines()] == [r["output"] for r in recs]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_forty_requests_decode_together(disunex_dirs, dtype):
+    """Forty requests decode side by side as replays of a captured graph: in bfloat16 such a step deals
+    its (token, expert) pairs to the experts in tiles, inside the graph, padding rows and all."""
+    from tffinfer_amd import EngineOptions, LLMEngine
+    d = disunex_dirs["dxQ"]
+    V = read_config(d)["vocab"]
+    prompts = [random_tokens(3 + i % 5, V, 500 + i) for i in range(40)]
+    eng = LLMEngine.from_model_dir(d, EngineOptions(dtype=dtype, page_size=16, kv_tokens=40 * 32, max_num_seqs=40,
+                                                    max_model_len=64))
+    eng.keep_logits = True
+    res = eng.generate(prompts, max_new_tokens=8, ignore_eos=True)
+    assert eng.runner._graphs and max(eng.runner._graphs) >= 40
+    checked = 0
+    for r in res:
+        assert len(r.output) == 8
+        ref = oracle_logits(d, r.prompt + r.output)
+        margins = []
+        plain.forward(*plain.load(d), r.prompt + r.output, margins=margins)
+        close = torch.stack(margins).min(0).values < MIN_MARGIN
+        for i, (row, tok) in enumerate(zip(r.logits, r.output)):
+            assert tok == int(torch.argmax(row))
+            if dtype == "bfloat16" and bool(close[:len(r.prompt) + i].any()):
+                break
+            assert rel_err(row, ref[len(r.prompt) + i - 1]) <= tol(dtype, d), f"request {r.prompt}: output {i}"
+            checked += 1
+    assert checked > 200
