@@ -217,16 +217,17 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 
 // ------------------------------------------------------------- many tokens: by expert ---
 // With many tokens a step the (token, expert) pairs are dealt to their experts first: every
-// expert's pairs fill tiles of 64 rows (128 where the experts have a few hundred pairs each) (the last one padded), so that a tile's rows share the
-// expert's matrices and the products run on the matrix cores.  A pair's row is computed from
-// the pair alone, k ascending, whatever tile and place it lands in: the result does not depend
-// on what else the step holds, nor on the order the pairs were dealt in.
+// expert's pairs fill tiles of `rows` pairs (64, or 128 where the experts have a few hundred pairs
+// each; an expert's last tile is padded), so that a tile's rows share the expert's matrices and the
+// products run on the matrix cores.  A pair's row is computed from the pair alone, k ascending,
+// whatever tile and place it lands in: the result does not depend on what else the step holds, nor
+// on the order the pairs were dealt in.
 //
-// tff_experts_sort:     tile_expert[tile], tile_rows[tile * 64 + i] = pair (token * top + k) or -1,
-//                       num_tiles[0]; one block.  At most pairs / 64 + E tiles.
-// tff_experts_gate_up_tiles / tff_experts_down_tiles: the two products per tile.  The down
-//                       product writes out[k][t][:] = wts[t][k] * Wd y: `top` planes that the
-//                       norm after the feed-forward adds up in the order of k.
+// experts_sort_kernel:  tile_expert[tile], tile_rows[tile * rows + i] = pair (token * top + k) or -1,
+//                       num_tiles[0]; one block.  At most pairs / rows + E tiles.
+// experts_tiles_kernel: the two products per tile.  The down product writes
+//                       out[k][t][:] = wts[t][k] * Wd y: `top` planes that the norm after the
+//                       feed-forward adds up in the order of k.
 
 __global__ __launch_bounds__(1024) void experts_sort_kernel(const int32_t* __restrict__ idx, int pairs, int E,
                                                             int rows, int32_t* __restrict__ tile_expert,
