@@ -201,7 +201,8 @@ class CacheManager:
         """``n_new`` tokens have been written.  Gives back the pages of window
         groups that no later query can reach: a query at position p >= count
         reads keys j >= p - window + 1, so block b is dead once
-        (b + 1) * page_size <= count - window + 1."""
+        (b + 1) * page_size <= count - window + 1; the blocks of the group's first
+        ``keep_first`` tokens stay."""
         st = self.requests[req]
         st.num_tokens += n_new
         ps = self.page_size
@@ -212,11 +213,12 @@ class CacheManager:
             w = g.spec.window
             if w > 0:
                 dead = max(0, (st.num_tokens - w + 1) // ps)
+                kept = -(-g.spec.keep_first // ps)      # blocks that hold tokens every later token reads
                 table = g.tables[req]
-                gone = [table[b] for b in range(min(dead, len(table))) if table[b] >= 0]
+                gone = [table[b] for b in range(kept, min(dead, len(table))) if table[b] >= 0]
                 if gone:
                     g.pool.free(gone)
-                    for b in range(min(dead, len(table))):
+                    for b in range(kept, min(dead, len(table))):
                         table[b] = -1
 
     def release(self, req) -> None:

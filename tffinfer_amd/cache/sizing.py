@@ -37,17 +37,20 @@ def state_bytes(requirements, max_seqs: int) -> int:
     return total
 
 
-def min_window_pages(window: int, page_size: int) -> int:
+def min_window_pages(window: int, page_size: int, keep_first: int = 0) -> int:
     """Pages a request must be able to hold in a group with a window to advance by one token:
-    the window's tokens, wherever the window's start falls in its page."""
-    return -(-max(window - 1, 0) // page_size) + 1
+    the window's tokens, wherever the window's start falls in its page, and the pages of the
+    first tokens that the group keeps for good."""
+    return -(-max(window - 1, 0) // page_size) + 1 + -(-keep_first // page_size)
 
 
-def window_pool_pages(window: int, page_size: int, max_seqs: int, token_budget: int) -> int:
+def window_pool_pages(window: int, page_size: int, max_seqs: int, token_budget: int, keep_first: int = 0) -> int:
     """Pages with which a group with a window never runs short: a request that brings n tokens to
     a step touches the n + window - 1 tokens that end with them, at most ceil((n + window - 1) /
-    page) + 1 pages, and a step's portions hold ``token_budget`` tokens between them."""
-    return max_seqs * (-(-max(window - 1, 0) // page_size) + 2) + -(-token_budget // page_size)
+    page) + 1 pages, and a step's portions hold ``token_budget`` tokens between them; every
+    request also keeps the pages of its first ``keep_first`` tokens."""
+    return (max_seqs * (-(-max(window - 1, 0) // page_size) + 2 + -(-keep_first // page_size))
+            + -(-token_budget // page_size))
 
 
 def bytes_per_page(spec: KVCacheSpec, layers: int, page_size: int, elem_size: int) -> int:
@@ -70,7 +73,7 @@ def plan_pages(requirements, page_size: int, elem_size: int, max_seqs: int, toke
     pages = {}
     for s in groups:
         if s.window > 0:
-            n = window_pool_pages(s.window, page_size, max_seqs, token_budget)
+            n = window_pool_pages(s.window, page_size, max_seqs, token_budget, s.keep_first)
             pages[s] = n if want_full is None else min(n, want_full)
     budget = None
     if kv_bytes is not None:

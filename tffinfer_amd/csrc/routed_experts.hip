@@ -2,9 +2,11 @@
 //
 // tff_route_topk:   z = Wr h in float32 (or given: a product that ran before), s = sigmoid(z); the `top` experts with the largest
 //                   s + bias are chosen (the lowest index among equals), their weights are
-//                   s / (sum of the chosen s + 1e-20): the bias moves the choice only.
+//                   s / (sum of the chosen s + 1e-20): the bias moves the choice only.  With `softmax`,
+//                   s = softmax(z) over all experts and the weights are the chosen s as they are.
 // tff_experts_gate_up: for every (token, chosen expert): g = min(Wg h, limit),
-//                   u = clamp(Wu h, -limit, limit), y = g * sigmoid(act_alpha * g) * (u + 1).
+//                   u = clamp(Wu h, -limit, limit), y = g * sigmoid(act_alpha * g) * (u + up_offset)
+//                   (limit = infinity, act_alpha = 1, up_offset = 0: silu(g) * u).
 // tff_experts_down: out[t] = sum over the token's experts, in the order they were chosen, of
 //                   weight * (Wd y), float32.
 //
@@ -56,31 +58,50 @@ __global__ __launch_bounds__(64 * RT_WAVES) void route_topk_kernel(const T* __re
                                                                    const float* __restrict__ Wr,
                                                                    const float* __restrict__ logits,
                                                                    const float* __restrict__ bias, int width, int E,
-                                                                   int top, int32_t* __restrict__ idx,
+                                                                   int top, int softmax, int32_t* __restrict__ idx,
                                                                    float* __restrict__ wts) {
     __shared__ float s_all[RT_MAX_E];
     __shared__ float c_all[RT_MAX_E];
     __shared__ int chosen[64];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     if (logits) {
-        for (int e = threadIdx.x; e < E; e += blockDim.x) {
-            const float s = 1.0f / (1.0f + expf(-logits[(size_t)t * E + e]));
-            s_all[e] = s;
-            c_all[e] = s + (bias ? bias[e] : 0.f);
-        }
+        for (int e = threadIdx.x; e < E; e += blockDim.x) s_all[e] = logits[(size_t)t * E + e];
     } else {
         const T* hr = h + (size_t)t * h_row;
         for (int e = wv; e < E; e += RT_WAVES) {
             const float z = wave_dot(hr, Wr + (size_t)e * width, width, lane);
-            if (lane == 0) {
-                const float s = 1.0f / (1.0f + expf(-z));
-                s_all[e] = s;
-                c_all[e] = s + (bias ? bias[e] : 0.f);
-            }
+            if (lane == 0) s_all[e] = z;
         }
     }
     __syncthreads();
     if (wv > 0) return;
+    // (one wave from here on: LDS works through its accesses in order)
+    if (softmax) {
+        // s = exp(z - max) / sum over all experts, the sum in the order of the lanes' strides and a tree
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s_all[e]);
+        mx = wave_max(mx);
+        float den = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float x = expf(s_all[e] - mx);
+            s_all[e] = x;
+            den += x;
+        }
+        den = wave_sum(den);
+        for (int e = lane; e < E; e += 64) {
+            const float s = s_all[e] / den;
+            s_all[e] = s;
+            c_all[e] = s + (bias ? bias[e] : 0.f);
+        }
+    } else {
+        for (int e = lane; e < E; e += 64) {
+            const float s = 1.0f / (1.0f + expf(-s_all[e]));
+            s_all[e] = s;
+            c_all[e] = s + (bias ? bias[e] : 0.f);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+    __builtin_amdgcn_wave_barrier();
     float sum = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
@@ -105,12 +126,12 @@ __global__ __launch_bounds__(64 * RT_WAVES) void route_topk_kernel(const T* __re
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
         __builtin_amdgcn_wave_barrier();
     }
-    const float inv = 1.0f / (sum + 1e-20f);
+    const float inv = softmax ? 1.0f : 1.0f / (sum + 1e-20f);
     if (lane < top) wts[(size_t)t * top + lane] = s_all[chosen[lane]] * inv;
 }
 
 TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
-                           int width, int E, int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream) {
+                           int width, int E, int top, int softmax, int32_t* idx, float* wts, int dtype, tff_stream_t stream) {
     TFF_REQUIRE(idx && wts && (logits || (h && Wr)), "route_topk: null pointer");
     TFF_REQUIRE(T >= 0 && (logits || (width > 0 && h_row >= width)), "route_topk: bad sizes T=%d width=%d row=%d", T, width, h_row);
     TFF_REQUIRE(E > 0 && E <= RT_MAX_E && top > 0 && top <= E && top <= 64,
@@ -118,9 +139,9 @@ TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const floa
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TFF_F32)
-        route_topk_kernel<float><<<T, 64 * RT_WAVES, 0, s>>>((const float*)h, h_row, Wr, logits, bias, width, E, top, idx, wts);
+        route_topk_kernel<float><<<T, 64 * RT_WAVES, 0, s>>>((const float*)h, h_row, Wr, logits, bias, width, E, top, softmax, idx, wts);
     else if (dtype == TFF_BF16)
-        route_topk_kernel<bf16_t><<<T, 64 * RT_WAVES, 0, s>>>((const bf16_t*)h, h_row, Wr, logits, bias, width, E, top, idx, wts);
+        route_topk_kernel<bf16_t><<<T, 64 * RT_WAVES, 0, s>>>((const bf16_t*)h, h_row, Wr, logits, bias, width, E, top, softmax, idx, wts);
     else
         return tff_fail("route_topk: unknown dtype %d", dtype);
     return tff_check_launch("route_topk");
@@ -132,7 +153,7 @@ TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const floa
 template <typename T>
 __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
     const T* __restrict__ h, int h_row, const T* __restrict__ Wg, const T* __restrict__ Wu,
-    const int32_t* __restrict__ idx, int top, int width, int ff, int ldw, float limit, float act_alpha,
+    const int32_t* __restrict__ idx, int top, int width, int ff, int ldw, float limit, float act_alpha, float up_offset,
     T* __restrict__ y) {
     const int pair = blockIdx.x;                  // token * top + k
     const int t = pair / top;
@@ -150,7 +171,7 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_gate_up_kernel(
         if (lane == 0) {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
-            const float a = g * (1.0f / (1.0f + expf(-act_alpha * g))) * (u + 1.0f);
+            const float a = g * (1.0f / (1.0f + expf(-act_alpha * g))) * (u + up_offset);
             y[(size_t)pair * ff + f] = from_f32<T>(a);
         }
     }
@@ -176,7 +197,7 @@ __global__ __launch_bounds__(64 * EX_WAVES) void experts_down_kernel(
 }
 
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, void* y,
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset, void* y,
                                 int dtype, tff_stream_t stream) {
     TFF_REQUIRE(h && Wg && Wu && idx && y, "experts_gate_up: null pointer");
     TFF_REQUIRE(T >= 0 && top > 0 && E > 0 && width > 0 && ff > 0 && h_row >= width && ldw >= width,
@@ -187,11 +208,11 @@ TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const 
     TFF_REQUIRE(grid.y <= 65535, "experts_gate_up: too many outputs");
     if (dtype == TFF_F32)
         experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, 0, s>>>((const float*)h, h_row, (const float*)Wg, (const float*)Wu,
-                                                                    idx, top, width, ff, ldw, limit, act_alpha, (float*)y);
+                                                                    idx, top, width, ff, ldw, limit, act_alpha, up_offset, (float*)y);
     else if (dtype == TFF_BF16)
         experts_gate_up_kernel<bf16_t><<<grid, 64 * EX_WAVES, 0, s>>>((const bf16_t*)h, h_row, (const bf16_t*)Wg,
                                                                      (const bf16_t*)Wu, idx, top, width, ff, ldw, limit,
-                                                                     act_alpha, (bf16_t*)y);
+                                                                     act_alpha, up_offset, (bf16_t*)y);
     else
         return tff_fail("experts_gate_up: unknown dtype %d", dtype);
     return tff_check_launch("experts_gate_up");
@@ -291,7 +312,7 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
     const bf16_t* __restrict__ a_rows, int a_row, const bf16_t* __restrict__ W0, const bf16_t* __restrict__ W1,
     const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_rows,
     const int32_t* __restrict__ num_tiles, const float* __restrict__ wts, int T, int top, int K, int N,
-    float limit, float act_alpha, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
+    float limit, float act_alpha, float up_offset, bf16_t* __restrict__ y, float* __restrict__ out, int max_tiles, int col_blocks,
     int ldw) {
     constexpr int ROWS = AFR * 16;       // pairs of a tile: 64, or 128 where the experts have many pairs each
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * AFR * 512];      // two sub-steps of AFR fragments
@@ -382,7 +403,7 @@ __global__ __launch_bounds__(256) void experts_tiles_kernel(
                 if (pair >= 0 && f < N) {
                     const float gv = fminf(g4[c], limit);
                     const float uv = fminf(fmaxf(u4[c], -limit), limit);
-                    y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + 1.0f));
+                    y[(size_t)pair * N + f] = (bf16_t)(gv * (1.0f / (1.0f + expf(-act_alpha * gv))) * (uv + up_offset));
                 }
             }
         } else {
@@ -410,7 +431,7 @@ TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row) {
 // y [T * top, ff] bfloat16; out float32 [top, T, width].  max_tiles >= T * top / 64 + E.
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
-                                 int ldw_in, int ldw_down, float limit, float act_alpha, int32_t* tile_expert,
+                                 int ldw_in, int ldw_down, float limit, float act_alpha, float up_offset, int32_t* tile_expert,
                                  int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
                                  tff_stream_t stream) {
     TFF_REQUIRE(h && Wg && Wu && Wd && idx && wts && tile_expert && tile_rows && num_tiles && y && out,
@@ -438,18 +459,18 @@ TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const
 #define EXT_LAUNCH(GU, AFRV, CB, ...) experts_tiles_kernel<GU, AFRV><<<((CB) + 7) / 8 * 8 * max_tiles, 256, 0, s>>>(__VA_ARGS__)
     if (tall)
         EXT_LAUNCH(true, 8, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     else
         EXT_LAUNCH(true, 4, cb_up, (const bf16_t*)h, h_row, (const bf16_t*)Wg, (const bf16_t*)Wu, tile_expert, tile_rows,
-                   num_tiles, wts, T, top, width, ff, limit, act_alpha, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
+                   num_tiles, wts, T, top, width, ff, limit, act_alpha, up_offset, (bf16_t*)y, nullptr, max_tiles, cb_up, ldw_in);
     rc = tff_check_launch("experts_gate_up_tiles");
     if (rc) return rc;
     if (tall)
         EXT_LAUNCH(false, 8, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
-                   T, top, ff, width, limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
+                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
     else
         EXT_LAUNCH(false, 4, cb_down, (const bf16_t*)y, ff, (const bf16_t*)Wd, nullptr, tile_expert, tile_rows, num_tiles, wts,
-                   T, top, ff, width, limit, act_alpha, nullptr, out, max_tiles, cb_down, ldw_down);
+                   T, top, ff, width, limit, act_alpha, up_offset, nullptr, out, max_tiles, cb_down, ldw_down);
 #undef EXT_LAUNCH
     return tff_check_launch("experts_down_tiles");
 }

@@ -256,13 +256,13 @@ TFF_API int tff_gelu(const void* x, void* out, int64_t n, int tanh_form, int dty
 // ---- routed experts (routed_experts.hip) ----
 // Router: s = sigmoid(z), z = Wr h in float32 (Wr [E, width] float32), or z = logits [T, E] where given
 // (h and Wr may then be null); the `top` largest s + bias (bias may be null) are chosen; idx [T, top],
-// wts [T, top] = s / (sum of the chosen s + 1e-20).
+// wts [T, top] = s / (sum of the chosen s + 1e-20).  softmax != 0: s = softmax(z) over all experts, wts = the chosen s.
 TFF_API int tff_route_topk(const void* h, int h_row, const float* Wr, const float* logits, const float* bias, int T,
-                           int width, int E, int top, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
-// y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + 1), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
+                           int width, int E, int top, int softmax, int32_t* idx, float* wts, int dtype, tff_stream_t stream);
+// y[(t, k), :] = g * sigmoid(act_alpha * g) * (u + up_offset), g = min(Wg[e] h_t, limit), u = clamp(Wu[e] h_t, +-limit),
 // e = idx[t, k]; Wg, Wu [E, ff, width], rows ldw elements apart.
 TFF_API int tff_experts_gate_up(const void* h, int h_row, const void* Wg, const void* Wu, const int32_t* idx, int T,
-                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, void* y,
+                                int top, int E, int width, int ff, int ldw, float limit, float act_alpha, float up_offset, void* y,
                                 int dtype, tff_stream_t stream);
 // out[t, :] = sum_k wts[t, k] * Wd[idx[t, k]] y[(t, k), :]; Wd [E, width, ff], rows ldw elements apart; out float32.
 TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, const float* wts, int T, int top, int E,
@@ -276,9 +276,52 @@ TFF_API int tff_experts_down(const void* y, const void* Wd, const int32_t* idx, 
 TFF_API int tff_experts_tiles_supported(int width, int ff, int h_row);
 TFF_API int tff_experts_by_tiles(const void* h, int h_row, const void* Wg, const void* Wu, const void* Wd,
                                  const int32_t* idx, const float* wts, int T, int top, int E, int width, int ff,
-                                 int ldw_in, int ldw_down, float limit, float act_alpha, int32_t* tile_expert,
+                                 int ldw_in, int ldw_down, float limit, float act_alpha, float up_offset, int32_t* tile_expert,
                                  int32_t* tile_rows, int32_t* num_tiles, int max_tiles, void* y, float* out,
                                  tff_stream_t stream);
+
+// ---- norms on a sublayer's output, sums over the model's depth (group_norm.hip) ----
+// y = delta row (planes added up first; row rows[r] where rows is given) cut into `groups` equal parts, each
+// divided by its own sqrt(mean(part^2) + eps), times w.  With resid: resid[r] += y and out[r] (optional) = the
+// new row; without: out[r] = y.
+TFF_API int tff_group_rmsnorm_add(float* resid, const float* delta, int planes, size_t plane, const int32_t* rows,
+                                  const float* w, int groups, float eps, void* out, int n, int H, int out_dtype,
+                                  tff_stream_t stream);
+// hist [>= n levels, `level` elements apart]: hist[n - 1] <- x; x <- sum_{j < n} coef[j] * hist[j]; out (optional) = x.
+TFF_API int tff_depth_average(float* hist, size_t level, int n, const float* coef, float* x, void* out, size_t count,
+                              int out_dtype, tff_stream_t stream);
+TFF_API int tff_scale_rows(float* x, float alpha, size_t count, tff_stream_t stream);
+
+// ---- a linear recurrence with a matrix of state per head (wkv.hip) ----
+// out [M, T, W] = x[t] + (x'[t] - x[t]) * mu[m]; x' the row before t in its request, for the first row of a
+// request's portion state[slot, prev_off : prev_off + W].
+TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state_row, size_t prev_off, const float* mu,
+                                int M, const int32_t* token_req, const int32_t* cu_tokens, const int32_t* state_slots,
+                                void* out, int T, int W, int out_dtype, tff_stream_t stream);
+// r, k, v, z float32 [T, >= H * D] with rows `row` elements apart; w = exp(-exp(z + w0)); per request (cu_tokens,
+// state_slots) and head, state[slot, h] = S [D, D]: o_t = (S + diag(u) k v^T)^T r, S <- diag(w) S + k v^T.
+// o float32 [T, H * D].  x (optional) [T, W]: the portion's last row goes to state[slot, prev_off : prev_off + W].
+TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, const float* z, size_t row, const float* w0,
+                               const float* u, float* state, size_t state_row, const int32_t* cu_tokens,
+                               const int32_t* state_slots, float* o, int R, int H, int D, const float* x, int W,
+                               size_t prev_off, tff_stream_t stream);
+// out = o / sqrt(mean over each head of o^2 + eps) * nw * silu(g); g rows g_row elements apart.
+TFF_API int tff_head_norm_gate(const float* o, const float* g, size_t g_row, const float* nw, float eps, void* out, int T,
+                               int H, int D, int out_dtype, tff_stream_t stream);
+TFF_API int tff_tanh(const float* in, void* out, size_t count, int out_dtype, tff_stream_t stream);
+
+// ---- attention whose heads exchange their scores (mixed_attention.hip) ----
+TFF_API int tff_qk_bias_norm_store(const float* qk, size_t row, const float* qb, const float* kb, float eps, void* q_out,
+                                   void* k_cache, void* v_cache, const int32_t* slot_mapping, int page_size, int T, int H,
+                                   int G, int D, int dtype, tff_stream_t stream);
+TFF_API int tff_mixed_attention_supported(int H, int D, int has_mix);
+// bias float32 [bias_rows, H] by distance (the last row for all larger distances) or null; mix float32 [H, H] or
+// null; cap 0: no soft cap; window 0: every earlier key; sink 0 / 1.
+TFF_API int tff_mixed_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                int bt_width, const int32_t* token_req, const int32_t* positions, const float* bias,
+                                int bias_rows, const float* mix, float scale, float cap, int window, int keep_first,
+                                int sink, void* out, int T, int H, int G, int D, int page_size, int dtype,
+                                tff_stream_t stream);
 
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

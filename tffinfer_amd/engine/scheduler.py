@@ -134,7 +134,7 @@ class Scheduler:
         for g in self.cache.groups:
             # a group with a window must hold what one more token touches; portions are cut to
             # what the free pages hold (_fit), so no larger bound is needed for the request to run
-            need = pages if g.spec.window <= 0 else min(pages, min_window_pages(g.spec.window, ps))
+            need = pages if g.spec.window <= 0 else min(pages, min_window_pages(g.spec.window, ps, g.spec.keep_first))
             if need > g.pool.num_pages:
                 raise RequestRefused(
                     f"request {req.id!r} needs {need} cache pages, the pool has {g.pool.num_pages} in all")

@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 
 
 class KernelLibraryError(RuntimeError):
@@ -50,10 +50,20 @@ _SIGNATURES = {
     "tff_head_linear": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P, _I, _P, _I, _P],
     "tff_scale_add_rmsnorm": [_P, _P, _I, _Z, _F, _P, _F, _P, _I, _I, _I, _P],
     "tff_gelu": [_P, _P, c_int64, _I, _I, _P],
-    "tff_route_topk": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P],
-    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P, _I, _P],
+    "tff_route_topk": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
+    "tff_experts_gate_up": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _I, _P],
     "tff_experts_tiles_supported": [_I, _I, _I],
-    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _P, _P, _I, _P, _P, _P],
+    "tff_experts_by_tiles": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P, _P, _P, _I, _P, _P, _P],
+    "tff_group_rmsnorm_add": [_P, _P, _I, _Z, _P, _P, _I, _F, _P, _I, _I, _I, _P],
+    "tff_depth_average": [_P, _Z, _I, _P, _P, _P, _Z, _I, _P],
+    "tff_scale_rows": [_P, _F, _Z, _P],
+    "tff_token_shift_mix": [_P, _P, _Z, _Z, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P],
+    "tff_wkv_recurrence": [_P, _P, _P, _P, _Z, _P, _P, _P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _Z, _P],
+    "tff_head_norm_gate": [_P, _P, _Z, _P, _F, _P, _I, _I, _I, _I, _P],
+    "tff_tanh": [_P, _P, _Z, _I, _P],
+    "tff_qk_bias_norm_store": [_P, _Z, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "tff_mixed_attention_supported": [_I, _I, _I],
+    "tff_mixed_attention": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _F, _F, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tff_experts_down": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],

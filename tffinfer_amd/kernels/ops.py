@@ -1019,10 +1019,11 @@ def gelu(x: torch.Tensor, tanh_form: bool = False) -> torch.Tensor:
 
 
 def route_topk(h: torch.Tensor | None, router: torch.Tensor | None, bias: torch.Tensor | None, top: int,
-               logits: torch.Tensor | None = None):
+               logits: torch.Tensor | None = None, softmax: bool = False):
     """s = sigmoid(z) with z = h . router^T in float32 (router float32 [E, width]) or z = ``logits``
     (float32 [T, E], a product that ran before); the ``top`` experts with the largest s + bias;
-    returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20))."""
+    returns (int32 [T, top], float32 [T, top] = s / (sum of the chosen s + 1e-20)).  With
+    ``softmax``, s = softmax(z) over all experts and the weights are the chosen s as they are."""
     if logits is not None:
         _req(logits, "router logits", torch.float32, 2)
         T, E = logits.shape
@@ -1043,7 +1044,7 @@ def route_topk(h: torch.Tensor | None, router: torch.Tensor | None, bias: torch.
     wts = torch.empty(T, top, dtype=torch.float32, device=dev)
     _lib.check(_lib.load().tff_route_topk(None if logits is not None else h.data_ptr(), width,
                                           None if logits is not None else router.data_ptr(), _ptr(logits), _ptr(bias),
-                                          T, width, E, int(top), idx.data_ptr(), wts.data_ptr(), dtype_code(dt), _stream()))
+                                          T, width, E, int(top), 1 if softmax else 0, idx.data_ptr(), wts.data_ptr(), dtype_code(dt), _stream()))
     return idx, wts
 
 
@@ -1064,8 +1065,8 @@ EXPERT_TILES_MIN_TOKENS = 32
 
 def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                    idx: torch.Tensor, wts: torch.Tensor, limit: float, act_alpha: float,
-                   by_tiles: bool | None = None) -> torch.Tensor:
-    """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + 1) with
+                   by_tiles: bool | None = None, up_offset: float = 1.0) -> torch.Tensor:
+    """The weighted sum of each token's chosen experts: y = g sigmoid(act_alpha g) (u + up_offset) with
     g = min(Wg h, limit), u = clamp(Wu h, -limit, limit); out = sum_k wts[:, k] Wd y.
     ``w_gate``, ``w_up`` [E, ff, >= width], ``w_down`` [E, width, >= ff] of h's type (the last
     dimension may be wider than what is multiplied: see :func:`pad_expert_rows`).  float32
@@ -1097,15 +1098,229 @@ def routed_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_
         out = torch.empty(top, T, width, dtype=torch.float32, device=h.device)
         _lib.check(L.tff_experts_by_tiles(
             h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(),
-            T, top, E, width, ff, ld_in, ld_down, float(limit), float(act_alpha), tables.data_ptr(), tables[max_tiles:].data_ptr(),
+            T, top, E, width, ff, ld_in, ld_down, float(limit), float(act_alpha), float(up_offset), tables.data_ptr(), tables[max_tiles:].data_ptr(),
             tables[129 * max_tiles:].data_ptr(), max_tiles, y.data_ptr(), out.data_ptr(), _stream()))
         return out if top > 1 else out[0]
     _lib.check(L.tff_experts_gate_up(h.data_ptr(), width, w_gate.data_ptr(), w_up.data_ptr(), idx.data_ptr(), T, top, E,
-                                     width, ff, ld_in, float(limit), float(act_alpha), y.data_ptr(), dtype_code(h.dtype),
+                                     width, ff, ld_in, float(limit), float(act_alpha), float(up_offset), y.data_ptr(), dtype_code(h.dtype),
                                      _stream()))
     out = torch.empty(T, width, dtype=torch.float32, device=h.device)
     _lib.check(L.tff_experts_down(y.data_ptr(), w_down.data_ptr(), idx.data_ptr(), wts.data_ptr(), T, top, E, width, ff,
                                   ld_down, out.data_ptr(), dtype_code(h.dtype), _stream()))
+    return out
+
+
+def group_rmsnorm_add(resid: torch.Tensor | None, delta, weight: torch.Tensor, groups: int, eps: float,
+                      out_dtype: torch.dtype | None = None, rows: torch.Tensor | None = None):
+    """A norm on a sublayer's output: every row of ``delta`` is cut into ``groups`` equal parts, each
+    divided by its own root mean square, the whole times ``weight``.  With ``resid`` the result is
+    added into the float32 residual stream in place and the new rows are returned in ``out_dtype``
+    (None: nothing is returned); without, the normed rows themselves are returned (of the rows
+    ``rows`` only, where given).  ``delta`` may be what ``linear`` returns with ``partials=True``."""
+    if isinstance(delta, PendingProduct):
+        delta = delta.run()
+    if isinstance(delta, ScaledRows):
+        delta = delta.materialize()
+    _req(delta, "group_rmsnorm_add delta", torch.float32, 3 if delta.dim() == 3 else 2)
+    planes, plane = 1, 0
+    if delta.dim() == 3:
+        planes, plane = delta.shape[0], delta.stride(0)
+    n_src, H = delta.shape[-2:]
+    _req(weight, "group_rmsnorm_add weight", torch.float32, 1)
+    if weight.numel() != H or groups <= 0 or H % groups:
+        raise _lib.KernelError(f"group_rmsnorm_add: rows of {H}, weight of {weight.numel()}, {groups} groups")
+    n = n_src
+    if resid is not None:
+        _req(resid, "group_rmsnorm_add resid", torch.float32, 2)
+        if tuple(resid.shape) != (n_src, H) or rows is not None:
+            raise _lib.KernelError(f"group_rmsnorm_add: resid {tuple(resid.shape)} for delta {tuple(delta.shape)}")
+    elif rows is not None:
+        _req(rows, "group_rmsnorm_add rows", torch.int32, 1)
+        if planes != 1:
+            raise _lib.KernelError("group_rmsnorm_add: chosen rows of partial sums")
+        n = rows.numel()
+    if resid is None and out_dtype is None:
+        out_dtype = torch.float32
+    out = torch.empty(n, H, dtype=out_dtype, device=delta.device) if out_dtype is not None else None
+    _lib.check(_lib.load().tff_group_rmsnorm_add(
+        _ptr(resid), delta.data_ptr(), planes, plane, _ptr(rows), weight.data_ptr(), int(groups), float(eps), _ptr(out),
+        n, H, dtype_code(out_dtype) if out_dtype is not None else 0, _stream()))
+    return out
+
+
+def depth_average(hist: torch.Tensor, n: int, coef: torch.Tensor, x: torch.Tensor,
+                  out_dtype: torch.dtype | None = None):
+    """``hist[n - 1] <- x; x <- sum_{j < n} coef[j] * hist[j]`` on the float32 residual stream ``x``
+    [T, W], with ``hist`` [depths, T, W] the stream as the embedding and every layer so far left it;
+    returns the new x in ``out_dtype`` (None: nothing)."""
+    _req(hist, "depth_average hist", torch.float32, 3)
+    _req(x, "depth_average x", torch.float32, 2)
+    _req(coef, "depth_average coef", torch.float32, 1)
+    if tuple(hist.shape[1:]) != tuple(x.shape) or not 1 <= n <= hist.shape[0] or coef.numel() < n:
+        raise _lib.KernelError(f"depth_average: {n} levels of {tuple(hist.shape)} for x {tuple(x.shape)}, "
+                               f"{coef.numel()} coefficients")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    _lib.check(_lib.load().tff_depth_average(hist.data_ptr(), hist.stride(0), int(n), coef.data_ptr(), x.data_ptr(),
+                                             _ptr(out), x.numel(), dtype_code(out_dtype) if out_dtype is not None else 0,
+                                             _stream()))
+    return out
+
+
+def scale_rows(x: torch.Tensor, alpha: float) -> torch.Tensor:
+    """``x <- alpha * x`` in place on float32 rows."""
+    _req(x, "scale_rows x", torch.float32)
+    _lib.check(_lib.load().tff_scale_rows(x.data_ptr(), float(alpha), x.numel(), _stream()))
+    return x
+
+
+def _state_rows(state: torch.Tensor, what: str) -> int:
+    _req(state, what, torch.float32, 2)
+    return state.stride(0)
+
+
+def token_shift_mix(x: torch.Tensor, state: torch.Tensor, prev_off: int, mu: torch.Tensor, batch,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """out[m, t] = x[t] + (x'[t] - x[t]) * mu[m] with x' the row of the token before t in its request:
+    the row above, or for the first token of a request's portion ``state[slot, prev_off:prev_off + W]``
+    (float32 [slots, row])."""
+    _req(x, "token_shift_mix x", torch.float32, 2)
+    _req(mu, "token_shift_mix mu", torch.float32, 2)
+    T, W = x.shape
+    M = mu.shape[0]
+    row = _state_rows(state, "token_shift_mix state")
+    if mu.shape[1] != W or prev_off < 0 or prev_off + W > row:
+        raise _lib.KernelError(f"token_shift_mix: rows of {W}, mu {tuple(mu.shape)}, state rows of {row}")
+    out = torch.empty(M, T, W, dtype=out_dtype, device=x.device)
+    _lib.check(_lib.load().tff_token_shift_mix(x.data_ptr(), state.data_ptr(), row, int(prev_off), mu.data_ptr(), M,
+                                               batch.token_req.data_ptr(), batch.cu_tokens.data_ptr(),
+                                               batch.state_slots.data_ptr(), out.data_ptr(), T, W, dtype_code(out_dtype),
+                                               _stream()))
+    return out
+
+
+def wkv_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, w0: torch.Tensor,
+                   u: torch.Tensor, state: torch.Tensor, batch, H: int, D: int, x: torch.Tensor | None = None,
+                   prev_off: int = 0) -> torch.Tensor:
+    """The recurrence o_t = (S + diag(u) k_t v_t^T)^T r_t, S <- diag(w_t) S + k_t v_t^T with
+    w_t = exp(-exp(z_t + w0)) over each request's tokens of this step, per head; S [D, D] float32 lies at
+    the start of the request's row of ``state`` (float32 [slots, row]).  r, k, v, z float32 [T, H * D]
+    (columns of wider rows are fine, all with the same stride).  ``x`` [T, W]: each request's last row
+    of it is left at ``state[slot, prev_off:]``.  Returns o float32 [T, H * D]."""
+    T = r.shape[0]
+    HD = H * D
+    for t, nm in ((r, "r"), (k, "k"), (v, "v"), (z, "z")):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.float32 or t.dim() != 2 \
+                or tuple(t.shape) != (T, HD) or t.stride(1) != 1 or t.stride(0) != r.stride(0):
+            raise _lib.KernelError(f"wkv_recurrence {nm}: expected float32 [{T}, {HD}] with the rows' stride of r")
+    _req(w0, "wkv_recurrence w0", torch.float32, 1)
+    _req(u, "wkv_recurrence u", torch.float32, 1)
+    if w0.numel() != HD or u.numel() != HD:
+        raise _lib.KernelError(f"wkv_recurrence: w0 and u must hold {HD} elements")
+    row = _state_rows(state, "wkv_recurrence state")
+    W = 0
+    if x is not None:
+        _req(x, "wkv_recurrence x", torch.float32, 2)
+        W = x.shape[1]
+        if x.shape[0] != T or prev_off < HD * D or prev_off + W > row:
+            raise _lib.KernelError("wkv_recurrence: the state's row does not hold x behind the heads' matrices")
+    if HD * D > row:
+        raise _lib.KernelError(f"wkv_recurrence: state rows of {row} for {H} heads of {D} x {D}")
+    o = torch.empty(T, HD, dtype=torch.float32, device=r.device)
+    if T == 0:
+        return o
+    _lib.check(_lib.load().tff_wkv_recurrence(r.data_ptr(), k.data_ptr(), v.data_ptr(), z.data_ptr(), r.stride(0),
+                                              w0.data_ptr(), u.data_ptr(), state.data_ptr(), row,
+                                              batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), o.data_ptr(),
+                                              batch.num_reqs, H, D, _ptr(x), W, int(prev_off), _stream()))
+    return o
+
+
+def head_norm_gate(o: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, eps: float, H: int, D: int,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """``o / sqrt(mean over each head of o^2 + eps) * weight * silu(g)`` for o, g float32 [T, H * D]."""
+    _req(o, "head_norm_gate o", torch.float32, 2)
+    _req(weight, "head_norm_gate weight", torch.float32, 1)
+    T = o.shape[0]
+    if not isinstance(g, torch.Tensor) or g.dtype != torch.float32 or g.dim() != 2 or g.stride(1) != 1 \
+            or tuple(g.shape) != (T, H * D) or o.shape[1] != H * D or weight.numel() != H * D:
+        raise _lib.KernelError("head_norm_gate: o and g must be float32 [T, heads * dim]")
+    out = torch.empty(T, H * D, dtype=out_dtype, device=o.device)
+    _lib.check(_lib.load().tff_head_norm_gate(o.data_ptr(), g.data_ptr(), g.stride(0) if T > 1 else H * D,
+                                              weight.data_ptr(), float(eps), out.data_ptr(), T, H, D,
+                                              dtype_code(out_dtype), _stream()))
+    return out
+
+
+def tanh(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    _req(x, "tanh input", torch.float32)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _lib.check(_lib.load().tff_tanh(x.data_ptr(), out.data_ptr(), x.numel(), dtype_code(out_dtype), _stream()))
+    return out
+
+
+def qk_bias_norm_store(qk: torch.Tensor, q_bias, k_bias, eps: float, H: int, G: int, D: int, kv) -> torch.Tensor:
+    """q and k of one projection (float32 [T, (H + G) * D]) with their biases added; q divided by its root
+    mean square per head and returned in the cache's type [T, H * D]; k written to the token's slot
+    as projected (the value pages) and divided by its root mean square (the key pages)."""
+    _req(qk, "qk_bias_norm_store qk", torch.float32, 2)
+    T = qk.shape[0]
+    if qk.shape[1] != (H + G) * D:
+        raise _lib.KernelError(f"qk_bias_norm_store: rows of {qk.shape[1]} for {H} + {G} heads of {D}")
+    for b, n, nm in ((q_bias, H * D, "q bias"), (k_bias, G * D, "k bias")):
+        if b is not None:
+            _req(b, nm, torch.float32, 1)
+            if b.numel() != n:
+                raise _lib.KernelError(f"qk_bias_norm_store: {nm} of {b.numel()} elements, expected {n}")
+    _check_cache(kv.k_cache, kv.v_cache, G, D, "qk_bias_norm_store")
+    dt = kv.k_cache.dtype
+    q = torch.empty(T, H * D, dtype=dt, device=qk.device)
+    _req(kv.slot_mapping, "slot_mapping", torch.int32, 1)
+    if kv.slot_mapping.numel() < T:
+        raise _lib.KernelError("qk_bias_norm_store: fewer slots than tokens")
+    _lib.check(_lib.load().tff_qk_bias_norm_store(qk.data_ptr(), qk.stride(0), _ptr(q_bias), _ptr(k_bias), float(eps),
+                                                  q.data_ptr(), kv.k_cache.data_ptr(), kv.v_cache.data_ptr(),
+                                                  kv.slot_mapping.data_ptr(), kv.page_size, T, H, G, D, dtype_code(dt),
+                                                  _stream()))
+    return q
+
+
+def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: float, softcap: float = 0.0,
+                    bias: torch.Tensor | None = None, mix: torch.Tensor | None = None, window: int = 0,
+                    keep_first: int = 0, sink: bool = False) -> torch.Tensor:
+    """Causal attention over the paged cache whose heads exchange their scores before the softmax:
+    s_g = softcap * tanh(scale * q_g . k_g / softcap) (softcap 0: scale * q_g . k_g) + bias[min(i - j, rows - 1), g];
+    s'_h = sum_g mix[h, g] s_g; key j is visible to query i if j <= i and (i - j < window or j < keep_first)
+    (window 0: all j <= i); softmax over the visible keys, with one more term of 1 in the denominator
+    if ``sink``; the values are the value pages.  q [T, H * D] in the cache's type; bias float32 [rows, H];
+    mix float32 [H, H]."""
+    dt = kv.k_cache.dtype
+    _req(q, "mixed_attention q", dt, 2)
+    T = q.shape[0]
+    if q.shape[1] != H * D or H % G:
+        raise _lib.KernelError(f"mixed_attention: q {tuple(q.shape)} for {H} heads of {D} on {G} kv heads")
+    _check_cache(kv.k_cache, kv.v_cache, G, D, "mixed_attention")
+    L = _lib.load()
+    if not L.tff_mixed_attention_supported(H, D, 1 if mix is not None else 0):
+        raise _lib.KernelError(f"mixed_attention: {H} heads of {D} are more than a block holds")
+    rows = 0
+    if bias is not None:
+        _req(bias, "mixed_attention bias", torch.float32, 2)
+        rows = bias.shape[0]
+        if bias.shape[1] != H or rows < 1:
+            raise _lib.KernelError(f"mixed_attention: bias {tuple(bias.shape)} for {H} heads")
+    if mix is not None:
+        _req(mix, "mixed_attention mix", torch.float32, 2)
+        if tuple(mix.shape) != (H, H):
+            raise _lib.KernelError(f"mixed_attention: mix {tuple(mix.shape)} for {H} heads")
+    bt = _req(kv.block_tables, "block_tables", torch.int32, 2)
+    if batch.token_req.numel() < T or batch.positions.numel() < T:
+        raise _lib.KernelError("mixed_attention: the step's tables are shorter than q")
+    out = torch.empty(T, H * D, dtype=dt, device=q.device)
+    _lib.check(L.tff_mixed_attention(q.data_ptr(), kv.k_cache.data_ptr(), kv.v_cache.data_ptr(), bt.data_ptr(),
+                                     bt.shape[1], batch.token_req.data_ptr(), batch.positions.data_ptr(), _ptr(bias),
+                                     rows, _ptr(mix), float(scale), float(softcap), int(window), int(keep_first),
+                                     1 if sink else 0, out.data_ptr(), T, H, G, D, kv.page_size, dtype_code(dt),
+                                     _stream()))
     return out
 
 

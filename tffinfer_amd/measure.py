@@ -67,7 +67,7 @@ def decode_bytes(model, batch: int, context: float, esz: int = 2) -> float:
     for call in model.schedule:
         spec = model.blocks[call.layer].mixer.cache_spec()
         if spec is not None:
-            keys = min(context, spec.window) if spec.window > 0 else context
+            keys = min(context, spec.window + spec.keep_first) if spec.window > 0 else context
             kv += 2 * spec.num_kv_heads * spec.head_dim * esz * batch * keys
     return weights + kv
 

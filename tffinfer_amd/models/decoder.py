@@ -55,7 +55,7 @@ class DecoderModel:
         self.dtype = None
         self.device = None
         H, V = config.hidden_size, config.vocab_size
-        self.embedding = Embedding(V, H)
+        self.embedding = Embedding(V, H, scale=getattr(config, "embedding_scale", 1.0))
         self.blocks = []
         for spec in config.layer_specs():
             mixer = MIXERS.build(spec.mixer)

@@ -30,6 +30,9 @@ class WeightSpec:
     """Shape of a weight tensor and the law random weights follow:
     ``matrix`` N(0, 0.02), ``norm`` 1 + N(0, 0.1), ``norm_offset`` N(0, 0.1) (a norm weight
     stored around zero), ``vector`` N(0, 0.5), ``embedding`` N(0, 0.02).
+    ``unit_interval`` U(0, 1), ``decay_log`` U(-3, 0.5) (z of a decay exp(-exp(z))), ``depth_coef``
+    N(0, 0.2) with 1 added to the last element.  A dimension of ``shape`` may be None: the
+    tensor itself gives that size (random weights then need it from the part's arguments).
     ``optional``: a file may leave the tensor out, and the part then does without it."""
     shape: tuple
     init: str = "matrix"
@@ -39,10 +42,12 @@ class WeightSpec:
 @dataclass(frozen=True)
 class KVCacheSpec:
     """Cache need of a mixer that keeps keys and values per token.
-    ``window`` 0: all tokens are kept; > 0: only the last ``window``."""
+    ``window`` 0: all tokens are kept; > 0: only the last ``window``, and the first
+    ``keep_first`` tokens of the request, which every later token goes on reading."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

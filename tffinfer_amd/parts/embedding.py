@@ -7,14 +7,15 @@ from .base import Part, WeightSpec, to_device
 
 
 class Embedding(Part):
-    """x[t, :] = E[token[t], :], no scaling, into the float32 residual stream.
-    Reference: src/kernel/cpu/embedding.cpp:34-49 (a CPU lookup there)."""
+    """x[t, :] = scale * E[token[t], :] into the float32 residual stream (scale 1: the rows
+    as they are).  Reference: src/kernel/cpu/embedding.cpp:34-49 (a CPU lookup there)."""
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
+        self.scale = float(scale)
         self.weight = None
 
     def weight_specs(self):
@@ -24,7 +25,10 @@ class Embedding(Part):
         self.weight = to_device(weights["weight"], dtype, device)
 
     def forward(self, ctx, token_ids):
-        return ctx.ops.embed(self.weight, token_ids)
+        x = ctx.ops.embed(self.weight, token_ids)
+        if self.scale != 1.0:
+            ctx.ops.scale_rows(x, self.scale)       # (in float32; the table itself also serves a tied head)
+        return x
 
 
 class OutputHead(Part):

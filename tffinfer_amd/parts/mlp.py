@@ -19,22 +19,27 @@ class SwiGLU(FeedForward):
     #: the input is used by ``ops.linear`` and by nothing else
     input_goes_to_linear = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.names = tuple(names)       # how the files call gate, up and down
+        if len(self.names) != 3:
+            from ..config.base import ConfigError
+            raise ConfigError("swiglu: 'names' are the names of gate, up and down")
         self.w_gate_up = None
         self.w_down = None
 
     def weight_specs(self):
         H, I = self.hidden_size, self.intermediate_size
         return {
-            "gate_proj.weight": WeightSpec((I, H)),
-            "up_proj.weight": WeightSpec((I, H)),
-            "down_proj.weight": WeightSpec((H, I)),
+            self.names[0]: WeightSpec((I, H)),
+            self.names[1]: WeightSpec((I, H)),
+            self.names[2]: WeightSpec((H, I)),
         }
 
     def load_weights(self, weights, dtype, device):
-        gate, up = weights["gate_proj.weight"], weights["up_proj.weight"]
+        gate, up = weights[self.names[0]], weights[self.names[1]]
         if dtype == torch.bfloat16 and torch.device(device).type == "cuda":
             # bfloat16: gate and up rows interleaved in groups of 16 in one weight, so that one
             # product streams both and applies silu(gate) * up to its float32 accumulators
@@ -44,7 +49,7 @@ class SwiGLU(FeedForward):
         else:
             # float32: gate and up stacked to [2I, H]; the activation is a kernel of its own
             self.w_gate_up = to_device(torch.cat([gate, up], 0), dtype, device)
-        self.w_down = to_device(weights["down_proj.weight"], dtype, device)
+        self.w_down = to_device(weights[self.names[2]], dtype, device)
 
     def forward(self, ctx, x):
         gu = ctx.ops.linear(x, self.w_gate_up)
@@ -104,18 +109,24 @@ class RoutedExperts(FeedForward):
                   y = g * sigmoid(act_alpha * g) * (u + 1),  f_e = Wd y
         f = sum over the chosen e of w_e f_e
 
+    ``router_softmax``: s = softmax(Wr z) over all experts instead, and w_e = s_e as it is.
+    ``limit`` None: no clamp; ``up_offset`` 0 and ``act_alpha`` 1: y = silu(g) * u.
+
     The experts' matrices lie stacked, [experts, out, in], so that a kernel finds an expert's
     rows by its number."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
-                 limit: float, act_alpha: float = 1.702, correction: bool = True):
+                 limit: float | None, act_alpha: float = 1.702, correction: bool = True,
+                 router_softmax: bool = False, up_offset: float = 1.0):
+        self.router_softmax = bool(router_softmax)
+        self.up_offset = float(up_offset)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.num_experts = int(num_experts)
         self.top = int(top)
-        self.limit = float(limit)
+        self.limit = float("inf") if limit is None else float(limit)
         self.act_alpha = float(act_alpha)
         self.has_correction = bool(correction)
         if not 0 < self.top <= self.num_experts:
@@ -169,7 +180,9 @@ class RoutedExperts(FeedForward):
         x = ops.as_tensor(x)
         if self.router_w is not None:
             idx, wts = ops.route_topk(None, None, self.correction, self.top,
-                                      logits=ops.linear(x, self.router_w, out_dtype=torch.float32))
+                                      logits=ops.linear(x, self.router_w, out_dtype=torch.float32),
+                                      softmax=self.router_softmax)
         else:
-            idx, wts = ops.route_topk(x, self.router, self.correction, self.top)
-        return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha)
+            idx, wts = ops.route_topk(x, self.router, self.correction, self.top, softmax=self.router_softmax)
+        return ops.routed_experts(x, self.w_gate, self.w_up, self.w_down, idx, wts, self.limit, self.act_alpha,
+                                  up_offset=self.up_offset)

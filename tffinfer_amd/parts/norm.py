@@ -55,3 +55,43 @@ class RMSNorm(Norm):
     def forward(self, ctx, resid, delta, rows=None, for_linear=False):
         return ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, ctx.act_dtype, rows=rows,
                                    for_linear=for_linear)
+
+
+@register_norm("group_rmsnorm")
+class GroupRMSNorm(Norm):
+    """A row is cut into ``groups`` equal consecutive parts; each part is divided by its own
+    sqrt(mean(part^2) + eps); the whole is multiplied by w.  Sums, roots and products in float32.
+
+    ``forward_add`` is the norm of a block that norms a sublayer's *output* before the sum:
+    ``resid <- resid + norm(delta)``.  ``forward`` norms the stream itself (the model's last norm)."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float, groups: int = 1, optional: bool = False):
+        self.size = int(size)
+        self.eps = float(eps)
+        self.groups = int(groups)
+        self.optional = bool(optional)
+        if self.groups <= 0 or self.size % self.groups:
+            from ..config.base import ConfigError
+            raise ConfigError(f"group norm: rows of {self.size} do not divide into {self.groups} groups")
+        self.weight = None
+
+    def weight_specs(self):
+        return {"weight": WeightSpec((self.size,), "norm", optional=self.optional)}
+
+    def load_weights(self, weights, dtype, device):
+        self.weight = (weights["weight"].to(torch.float32).contiguous().to(device)
+                       if "weight" in weights else None)
+
+    def forward_add(self, ctx, resid, delta):
+        """``resid <- resid + norm(delta)`` in place; returns the new rows in the activation type
+        (the stream itself where that is float32)."""
+        out = ctx.ops.group_rmsnorm_add(resid, delta, self.weight, self.groups, self.eps,
+                                        None if ctx.act_dtype == torch.float32 else ctx.act_dtype)
+        return resid if out is None else out
+
+    def forward(self, ctx, resid, delta, rows=None, for_linear=False):
+        if delta is not None:
+            resid += ctx.ops.as_tensor(delta)
+        return ctx.ops.group_rmsnorm_add(None, resid, self.weight, self.groups, self.eps, ctx.act_dtype, rows=rows)

@@ -35,8 +35,12 @@ def check_weights(expected: dict[str, WeightSpec], found: dict[str, torch.Tensor
     """Raises one WeightError naming everything that is wrong."""
     missing = [n for n in expected if n not in found and not expected[n].optional]
     unexpected = [n for n in found if n not in expected and n not in ignorable]
+    def fits(want, got):
+        # (None: a size that the tensor itself gives, a table's rows for instance)
+        return len(want) == len(got) and all(w is None or w == g for w, g in zip(want, got))
+
     wrong_shape = [(n, expected[n].shape, tuple(found[n].shape)) for n in expected
-                   if n in found and tuple(found[n].shape) != tuple(expected[n].shape)]
+                   if n in found and not fits(tuple(expected[n].shape), tuple(found[n].shape))]
     wrong_dtype = [(n, found[n].dtype) for n in expected if n in found and found[n].dtype not in _FLOATS]
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(sorted(missing), sorted(unexpected), wrong_shape, wrong_dtype, where)

@@ -14,7 +14,7 @@ MATRIX_STD = 0.02
 NORM_STD = 0.1
 VECTOR_STD = 0.5
 #: laws whose tensors are kept in float32 whatever the matrices are stored in
-FLOAT32_INITS = ("norm", "norm_offset", "vector")
+FLOAT32_INITS = ("norm", "norm_offset", "vector", "unit_interval", "decay_log", "depth_coef")
 
 
 def tensor_seed(seed: int, name: str) -> int:
@@ -29,7 +29,17 @@ def random_tensor(spec: WeightSpec, seed: int, name: str, device="cpu") -> torch
     enter scores or logits (``vector``) N(0, 0.5)."""
     g = torch.Generator(device=device)
     g.manual_seed(tensor_seed(seed, name))
+    if any(n is None for n in spec.shape):
+        raise ValueError(f"random weights for '{name}': its shape {spec.shape} leaves a size open; "
+                         "give the part that size as an argument")
+    if spec.init in ("unit_interval", "decay_log"):
+        x = torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device)
+        return x if spec.init == "unit_interval" else 3.5 * x - 3.0
     x = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device)
+    if spec.init == "depth_coef":
+        x = 0.2 * x
+        x.view(-1)[-1] += 1.0
+        return x
     if spec.init == "norm":
         return 1.0 + NORM_STD * x
     if spec.init == "norm_offset":
