@@ -29,6 +29,14 @@ def disunex_dirs(tmp_path_factory):
     return {name: make_disunex_dir(str(base / name), cfg, seed) for name, (cfg, seed) in DISUNEX_CONFIGS.items()}
 
 
+@pytest.fixture(scope="session")
+def netovik_dirs(tmp_path_factory):
+    """Model folders of the tiny Netovik configurations (sharpened weights), once per session."""
+    from netovik_models import NETOVIK_CONFIGS, make_netovik_dir
+    base = tmp_path_factory.mktemp("netovik")
+    return {name: make_netovik_dir(str(base / name), cfg, seed) for name, (cfg, seed) in NETOVIK_CONFIGS.items()}
+
+
 @pytest.fixture(autouse=True)
 def _seeded():
     """Every test draws the same random inputs in every run."""

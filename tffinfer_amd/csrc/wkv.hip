@@ -55,12 +55,12 @@ TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state
     return tff_check_launch("token_shift_mix");
 }
 
-#define WKV_MAX_D 256
+#define WKV_MAX_D 128     // (a thread keeps a slice of a column of S in registers)
 #define WKV_MAX_SLICES 4
 
 // KPT key channels a thread; ceil(D / KPT) <= 4 slices of the key channels; thread = slice * D + value channel.
 template <int KPT>
-__global__ __launch_bounds__(1024) void wkv_recurrence_kernel(
+__global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
     const float* __restrict__ z, size_t row, const float* __restrict__ w0, const float* __restrict__ u,
     float* __restrict__ state, size_t state_row, const int32_t* __restrict__ cu_tokens,
@@ -143,8 +143,7 @@ TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, c
     wkv_recurrence_kernel<KPT><<<grid, D * ((D + KPT - 1) / KPT), 0, s>>>(r, k, v, z, row, w0, u, state, state_row, \
                                                                            cu_tokens, state_slots, o, H, D, x, W, prev_off)
     if (D <= 64) WKV_LAUNCH(16);
-    else if (D <= 128) WKV_LAUNCH(32);
-    else WKV_LAUNCH(64);
+    else WKV_LAUNCH(32);
 #undef WKV_LAUNCH
     return tff_check_launch("wkv_recurrence");
 }

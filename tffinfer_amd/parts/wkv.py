@@ -41,9 +41,9 @@ class WKVMixer(Mixer):
         self.head_dim = int(head_dim)
         self.norm_eps = float(norm_eps)
         self.decay_rank = None if decay_rank is None else int(decay_rank)
-        if self.hidden_size <= 0 or self.num_heads <= 0 or not 0 < self.head_dim <= 256:
+        if self.hidden_size <= 0 or self.num_heads <= 0 or not 0 < self.head_dim <= 128:
             raise ConfigError(f"wkv: {num_heads} heads of {head_dim} on rows of {hidden_size} "
-                              "(a head has up to 256 channels)")
+                              "(a head has up to 128 channels)")
         self.mu = self.w0 = self.u = self.norm = None
         self.w_r = self.w_k = self.w_v = self.w_g = self.w_w1 = self.w_w2 = self.w_o = None
 
