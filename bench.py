@@ -57,9 +57,37 @@ DISUNEX_SHAPES = {
 }
 
 
+def netovik_shape(width, wkv_heads, wkv_dim, heads, kv_heads, dim, window, keep_first, dense_ff, experts, top, expert_ff,
+                  layers, vocab=151936):
+    """A Netovik configuration of ``layers`` layers: two recurrence layers, then one of attention, and so
+    on; dense and routed feed-forwards in turn."""
+    rec = {"type": "wkv", "mixer": {"heads": wkv_heads, "dim": wkv_dim, "decay_rank": 64}}
+    att = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                          "softcap": 30.0, "bias_max": 512, "bias_buckets": 32,
+                                          "mask": {"size": window, "keep_first": keep_first}}}
+    mlps = [{"kind": "dense", "ff": dense_ff},
+            {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}]
+    return {"architecture": "Netovik", "width": width, "vocab": vocab, "norm": {"eps": 1e-6, "groups": 2},
+            "embedding": {"scale": 0.5},
+            "layers": [dict(att if i % 3 == 2 else rec, mlp=mlps[i % 2]) for i in range(layers)]}
+
+
+# Netovik at sizes that resemble a real model's layers, each beside the Qwen3 shape of the same width (the same
+# gated feed-forward; the recurrence's five projections and its output are six square matrices where the
+# attention of the Qwen3 shape has the q, k, v and o of grouped heads)
+NETOVIK_SHAPES = {
+    "2k": ("1.7b", dict(width=2048, wkv_heads=32, wkv_dim=64, heads=16, kv_heads=4, dim=128, window=1024, keep_first=4,
+                        dense_ff=6144, experts=16, top=2, expert_ff=1024)),
+    "4k": ("8b", dict(width=4096, wkv_heads=64, wkv_dim=64, heads=32, kv_heads=8, dim=128, window=1024, keep_first=4,
+                      dense_ff=12288, experts=32, top=4, expert_ff=1536)),
+}
+
+DESIGNS = {"disunex": ("Disunex", DISUNEX_SHAPES, disunex_shape), "netovik": ("Netovik", NETOVIK_SHAPES, netovik_shape)}
+
+
 def design_points(args):
-    """Prefill and decode throughput of the Disunex design at the sizes of DISUNEX_SHAPES, and of the
-    Qwen3 shape of the same width and number of layers beside it, one JSON line."""
+    """Prefill and decode throughput of a second design (--design) at the sizes of its table of shapes, and
+    of the Qwen3 shape of the same width and number of layers beside it, one JSON line."""
     import gc
     import torch
     from tffinfer_amd import EngineOptions, LLMEngine
@@ -70,13 +98,14 @@ def design_points(args):
     L = args.layers or 8
     T, batch, context = args.prefill_tokens, args.batch, args.context
     steps, warmup = min(args.steps, 32), min(args.warmup, 4)
-    out = {"design": "Disunex", "layers_run": L, "prefill_tokens": T, "decode_batch": batch, "decode_context": context,
+    design, shapes, make_shape = DESIGNS[args.design]
+    out = {"design": design, "layers_run": L, "prefill_tokens": T, "decode_batch": batch, "decode_context": context,
            "dtype": "bf16", "data": "synthetic (seeded random weights and token ids)", "shapes": {}}
-    which = [args.design_shape] if args.design_shape else sorted(DISUNEX_SHAPES)
+    which = [args.design_shape] if args.design_shape else sorted(shapes)
     for name in which:
-        beside, sizes = DISUNEX_SHAPES[name]
+        beside, sizes = shapes[name]
         row = {}
-        for label, cfg in (("disunex", disunex_shape(layers=L, **sizes)),
+        for label, cfg in ((args.design, make_shape(layers=L, **sizes)),
                            ("qwen3_" + beside, dict(SHAPES[beside][1], num_hidden_layers=L))):
             if args.design_only and label != args.design_only and not label.startswith(args.design_only):
                 continue
@@ -145,12 +174,12 @@ def parse_args():
                     help="with --mixed: the scheduler cuts steps a little over a multiple of this many tokens down "
                          "to the multiple (default: the engine's own, 256; 0: off)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--design", choices=["disunex"], default=None,
+    ap.add_argument("--design", choices=sorted(DESIGNS), default=None,
                     help="instead of the benchmark line: prefill (--prefill-tokens) and decode (--batch, --context) "
                          "throughput of this design at sizes that resemble a real model's layers, each beside the "
                          "Qwen3 shape of the same width, --layers layers each (default 8)")
     ap.add_argument("--design-shape", default=None, help="with --design: one of its sizes only (2k, 4k)")
-    ap.add_argument("--design-only", default=None, help="with --design: 'disunex' or 'qwen3' only (for profiling)")
+    ap.add_argument("--design-only", default=None, help="with --design: the design itself or 'qwen3' only (for profiling)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure streaming-read bandwidth, back-to-back MFMA rates and a large square product "
                          "on this machine and stop")

@@ -57,8 +57,13 @@ TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state
 
 #define WKV_MAX_D 128     // (a thread keeps a slice of a column of S in registers)
 #define WKV_MAX_SLICES 4
+#define WKV_CHUNK_ELEMS 1024   // tokens of a chunk x head size, at most
+#define WKV_EPT 4              // elements of a chunk's array a thread fetches, at most
 
 // KPT key channels a thread; ceil(D / KPT) <= 4 slices of the key channels; thread = slice * D + value channel.
+// The tokens of a portion pass in chunks of up to 16: a chunk's r, k, w, v are fetched into registers while the
+// chunk before it is worked through from LDS, so that no token waits for memory; within a chunk a token costs
+// its multiply-adds and one barrier (the slices' partial sums meet in LDS, in a buffer of the token's parity).
 template <int KPT>
 __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
@@ -66,13 +71,16 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     float* __restrict__ state, size_t state_row, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ state_slots, float* __restrict__ o, int H, int D, const float* __restrict__ x, int W,
     size_t prev_off) {
-    __shared__ float sr[2][WKV_MAX_D], sk[2][WKV_MAX_D], sw[2][WKV_MAX_D], su[WKV_MAX_D];
-    __shared__ float part[WKV_MAX_SLICES][WKV_MAX_D];
-    const int h = blockIdx.x, req = blockIdx.y, tid = threadIdx.x;
+    __shared__ float buf[2][4][WKV_CHUNK_ELEMS];       // r, k, w, v of a chunk, [token in chunk][channel]
+    __shared__ float so[WKV_CHUNK_ELEMS];
+    __shared__ float su[WKV_MAX_D];
+    __shared__ float part[2][WKV_MAX_SLICES][WKV_MAX_D];
+    const int h = blockIdx.x, req = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
     const int t0 = cu_tokens[req], t1 = cu_tokens[req + 1];
     if (t1 <= t0) return;
-    const int slices = blockDim.x / D;
+    const int slices = nt / D;
     const int vi = tid % D, ks = tid / D;
+    const int C = min(min(16, WKV_EPT * slices), WKV_CHUNK_ELEMS / D);      // tokens a chunk
     float* srow = state + (size_t)state_slots[req] * state_row;
     float* S = srow + (size_t)h * D * D;
     const size_t col = (size_t)h * D;
@@ -82,40 +90,69 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
         const int kk = ks * KPT + i;
         s[i] = kk < D ? S[(size_t)kk * D + vi] : 0.f;
     }
-    if (tid < D) {
-        su[tid] = u[col + tid];
-        const size_t a = (size_t)t0 * row + col + tid;
-        sr[0][tid] = r[a];
-        sk[0][tid] = k[a];
-        sw[0][tid] = expf(-expf(z[a] + w0[col + tid]));
-    }
-    for (int t = t0; t < t1; ++t) {
-        const int b = (t - t0) & 1;
-        __syncthreads();
-        const float vt = v[(size_t)t * row + col + vi];
-        float acc = 0.f;
+    if (tid < D) su[tid] = u[col + tid];
+    float fr[WKV_EPT], fk[WKV_EPT], fz[WKV_EPT], fv[WKV_EPT];
+    // a chunk's elements e = token * D + channel are dealt to the threads in strides of the block
+    auto fetch = [&](int base) {
+        const int n = min(C, t1 - base) * D;
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            const int kk = ks * KPT + i;
-            if (kk < D) {
-                const float kv = sk[b][kk] * vt;
-                acc = fmaf(sr[b][kk], fmaf(su[kk], kv, s[i]), acc);
-                s[i] = fmaf(sw[b][kk], s[i], kv);
+        for (int i = 0; i < WKV_EPT; ++i) {
+            const int e = tid + i * nt;
+            if (e < n) {
+                const size_t a = (size_t)(base + e / D) * row + col + e % D;
+                fr[i] = r[a];
+                fk[i] = k[a];
+                fz[i] = z[a] + w0[col + e % D];
+                fv[i] = v[a];
             }
         }
-        part[ks][vi] = acc;
-        if (t + 1 < t1 && tid < D) {
-            const size_t a = (size_t)(t + 1) * row + col + tid;
-            sr[b ^ 1][tid] = r[a];
-            sk[b ^ 1][tid] = k[a];
-            sw[b ^ 1][tid] = expf(-expf(z[a] + w0[col + tid]));
+    };
+    auto stage = [&](int base, int b) {
+        const int n = min(C, t1 - base) * D;
+#pragma unroll
+        for (int i = 0; i < WKV_EPT; ++i) {
+            const int e = tid + i * nt;
+            if (e < n) {
+                buf[b][0][e] = fr[i];
+                buf[b][1][e] = fk[i];
+                buf[b][2][e] = expf(-expf(fz[i]));
+                buf[b][3][e] = fv[i];
+            }
+        }
+    };
+    fetch(t0);
+    stage(t0, 0);
+    int b = 0;
+    for (int base = t0; base < t1; base += C, b ^= 1) {
+        const int n = min(C, t1 - base);
+        __syncthreads();
+        if (base + C < t1) fetch(base + C);
+        for (int c = 0; c < n; ++c) {
+            const float* cr = buf[b][0] + c * D;
+            const float* ck = buf[b][1] + c * D;
+            const float* cw = buf[b][2] + c * D;
+            const float vt = buf[b][3][c * D + vi];
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < KPT; ++i) {
+                const int kk = ks * KPT + i;
+                if (kk < D) {
+                    const float kv = ck[kk] * vt;
+                    acc = fmaf(cr[kk], fmaf(su[kk], kv, s[i]), acc);
+                    s[i] = fmaf(cw[kk], s[i], kv);
+                }
+            }
+            part[c & 1][ks][vi] = acc;
+            __syncthreads();
+            if (ks == 0) {
+                float sum = part[c & 1][0][vi];
+                for (int p = 1; p < slices; ++p) sum += part[c & 1][p][vi];
+                so[c * D + vi] = sum;
+            }
         }
         __syncthreads();
-        if (ks == 0) {
-            float sum = part[0][vi];
-            for (int p = 1; p < slices; ++p) sum += part[p][vi];
-            o[(size_t)t * H * D + col + vi] = sum;
-        }
+        for (int e = tid; e < n * D; e += nt) o[(size_t)(base + e / D) * H * D + col + e % D] = so[e];
+        if (base + C < t1) stage(base + C, b ^ 1);
     }
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
@@ -124,7 +161,7 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     }
     if (h == 0 && x) {
         const float* last = x + (size_t)(t1 - 1) * W;
-        for (int c = tid; c < W; c += blockDim.x) srow[prev_off + c] = last[c];
+        for (int c = tid; c < W; c += nt) srow[prev_off + c] = last[c];
     }
 }
 

@@ -60,15 +60,20 @@ def prefill_flops(model, T: int) -> float:
 def decode_bytes(model, batch: int, context: float, esz: int = 2) -> float:
     """Bytes a decode step has to read, from the model's own parts: every matrix it multiplies
     with once (a layer that the run order names twice, twice), the output head, and the keys and
-    values that every layer call reads for the live requests (a window's worth where it has one)."""
+    values that every layer call reads for the live requests (a window's worth where it has one,
+    and the first tokens it keeps), or the state of fixed size that a mixer keeps per request."""
     cfg = model.config
     weights = (matrix_elements_per_step(model, batch, streamed=True) + cfg.hidden_size * cfg.vocab_size) * esz
     kv = 0.0
     for call in model.schedule:
-        spec = model.blocks[call.layer].mixer.cache_spec()
+        mixer = model.blocks[call.layer].mixer
+        spec = mixer.cache_spec()
         if spec is not None:
             keys = min(context, spec.window + spec.keep_first) if spec.window > 0 else context
             kv += 2 * spec.num_kv_heads * spec.head_dim * esz * batch * keys
+        state = mixer.state_spec()
+        if state is not None:       # (a request's state of fixed size is read whole at every token)
+            kv += batch * math.prod(state.shape) * state.dtype.itemsize
     return weights + kv
 
 
