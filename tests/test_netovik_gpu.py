@@ -108,7 +108,7 @@ def test_mixes_with_the_token_before():
         at += n
 
 
-@pytest.mark.parametrize("H,D", [(3, 8), (2, 24), (1, 40), (2, 64), (2, 128)])
+@pytest.mark.parametrize("H,D", [(3, 8), (2, 16), (2, 24), (1, 40), (2, 48), (2, 64), (1, 100), (2, 128)])
 def test_recurrence_whole_and_in_portions(H, D):
     """The recurrence over 70 tokens at once, and the same tokens in portions of 1 to 30 beside another
     request, with the state carried in a slot: the same numbers, bit for bit; decays from almost 0 to almost 1."""
@@ -297,7 +297,7 @@ def test_batches_of_unequal_requests_share_the_attention():
     lengths = [90, 41, 7]
     cases = [_attention_case(H, G, D, n, 20 + n) for n in lengths]
     qb, kb = cases[0][1], cases[0][2]
-    args = dict(scale=0.5, softcap=6.0, window=33, keep_first=2, sink=True)
+    args = dict(scale=0.5, softcap=6.0, window=33, keep_first=2, sink=True, splits=1)
     alone, cache = [], _Cache(G, D, page, lengths, torch.float32, seed=4)
     for r, (n, c) in enumerate(zip(lengths, cases)):
         kv = cache.view([r], [0], [n])
@@ -313,7 +313,11 @@ def test_batches_of_unequal_requests_share_the_attention():
     rows = torch.cat([c[0][f:] for c, f in zip(cases, firsts)], 0).contiguous().to(DEV)
     q = ops.qk_bias_norm_store(rows, qb.to(DEV), kb.to(DEV), eps, H, G, D, kv)
     got = ops.mixed_attention(q, H, G, D, kv, _batch(news, firsts), **args)
-    assert torch.equal(got, torch.cat([a[f:] for a, f in zip(alone, firsts)], 0))
+    want = torch.cat([a[f:] for a, f in zip(alone, firsts)], 0)
+    assert torch.equal(got, want)
+    # the keys of each token dealt to several blocks and merged: the same to rounding
+    for splits in (None, 2, 5):
+        assert _err(ops.mixed_attention(q, H, G, D, kv, _batch(news, firsts), **dict(args, splits=splits)), want) < 2e-6
 
 
 @pytest.mark.parametrize("E,top", [(8, 3), (2, 2), (5, 1), (70, 4)])

@@ -16,39 +16,57 @@
 
 #define GN_THREADS 256
 
+#define GN_ITS 8       // a group of up to 2048 elements passes through memory once
+
+// One block per (row, group).
 template <typename TO>
 __global__ __launch_bounds__(GN_THREADS) void group_rmsnorm_add_kernel(
     float* __restrict__ resid, const float* __restrict__ delta, int planes, size_t plane,
     const int32_t* __restrict__ rows, const float* __restrict__ w, int groups, float eps,
     TO* __restrict__ out, int H) {
     __shared__ float red[17];
-    const int r = blockIdx.x, tid = threadIdx.x;
+    const int r = blockIdx.x / groups, g = blockIdx.x % groups, tid = threadIdx.x;
     const int src = rows ? rows[r] : r;
-    const float* dl = delta + (size_t)src * H;
-    float* x = resid ? resid + (size_t)r * H : nullptr;
-    TO* o = out ? out + (size_t)r * H : nullptr;
-    const int Hg = H / groups;
-    for (int g = 0; g < groups; ++g) {
-        const int base = g * Hg;
-        float ss = 0.f;
-        for (int j = tid; j < Hg; j += GN_THREADS) {
-            float d = dl[base + j];
-            for (int p = 1; p < planes; ++p) d += dl[p * plane + base + j];
-            ss = fmaf(d, d, ss);
-        }
-        ss = block_sum(ss, red);
-        const float rr = 1.0f / sqrtf(ss / (float)Hg + eps);
-        for (int j = tid; j < Hg; j += GN_THREADS) {
-            float d = dl[base + j];
-            for (int p = 1; p < planes; ++p) d += dl[p * plane + base + j];
-            float y = d * rr * w[base + j];
-            if (x) {
-                y += x[base + j];
-                x[base + j] = y;
-            }
-            if (o) o[base + j] = from_f32<TO>(y);
+    const int Hg = H / groups, base = g * Hg;
+    const float* dl = delta + (size_t)src * H + base;
+    float* x = resid ? resid + (size_t)r * H + base : nullptr;
+    TO* o = out ? out + (size_t)r * H + base : nullptr;
+    const float* wg = w + base;
+    auto term = [&](int j) {
+        float d = dl[j];
+        for (int p = 1; p < planes; ++p) d += dl[p * plane + j];
+        return d;
+    };
+    float cache[GN_ITS];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < GN_ITS; ++it) {
+        const int j = tid + it * GN_THREADS;
+        if (j < Hg) {
+            cache[it] = term(j);
+            ss = fmaf(cache[it], cache[it], ss);
         }
     }
+    for (int j = tid + GN_ITS * GN_THREADS; j < Hg; j += GN_THREADS) {
+        const float d = term(j);
+        ss = fmaf(d, d, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rr = 1.0f / sqrtf(ss / (float)Hg + eps);
+    auto emit = [&](int j, float d) {
+        float y = d * rr * wg[j];
+        if (x) {
+            y += x[j];
+            x[j] = y;
+        }
+        if (o) o[j] = from_f32<TO>(y);
+    };
+#pragma unroll
+    for (int it = 0; it < GN_ITS; ++it) {
+        const int j = tid + it * GN_THREADS;
+        if (j < Hg) emit(j, cache[it]);
+    }
+    for (int j = tid + GN_ITS * GN_THREADS; j < Hg; j += GN_THREADS) emit(j, term(j));
 }
 
 TFF_API int tff_group_rmsnorm_add(float* resid, const float* delta, int planes, size_t plane, const int32_t* rows,
@@ -60,10 +78,10 @@ TFF_API int tff_group_rmsnorm_add(float* resid, const float* delta, int planes, 
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (!out || out_dtype == TFF_F32)
-        group_rmsnorm_add_kernel<float><<<n, GN_THREADS, 0, s>>>(resid, delta, planes, plane, rows, w, groups, eps,
+        group_rmsnorm_add_kernel<float><<<n * groups, GN_THREADS, 0, s>>>(resid, delta, planes, plane, rows, w, groups, eps,
                                                                   (float*)out, H);
     else if (out_dtype == TFF_BF16)
-        group_rmsnorm_add_kernel<bf16_t><<<n, GN_THREADS, 0, s>>>(resid, delta, planes, plane, rows, w, groups, eps,
+        group_rmsnorm_add_kernel<bf16_t><<<n * groups, GN_THREADS, 0, s>>>(resid, delta, planes, plane, rows, w, groups, eps,
                                                                    (bf16_t*)out, H);
     else
         return tff_fail("group_rmsnorm_add: unknown dtype %d", out_dtype);

@@ -12,9 +12,10 @@
 // tff_qk_bias_norm_store: q and k rows from one projection [T, (H + G) * D] (float32) get their biases;
 //   q is divided by its root mean square over the head and written out; k goes into the token's slot
 //   twice: as projected into the value page, divided by its root mean square into the key page.
-// tff_mixed_attention: one block per query token, all heads; keys in tiles of 64 whose borders are
-//   multiples of 64 from the sequence's start, so a query's sums are formed in the same order in
-//   every step that computes it.
+// tff_mixed_attention: one block per query token (and split of its keys), all heads; keys in tiles of 64
+//   whose borders are multiples of 64 from the sequence's start, so a query's sums are formed in the same
+//   order in every step that computes it with the same number of splits; a step of few tokens splits each
+//   token's tiles over several blocks and a second kernel puts them together.
 #include "common.h"
 #include "tffinfer_kernels.h"
 
@@ -74,8 +75,8 @@ TFF_API int tff_qk_bias_norm_store(const float* qk, size_t row, const float* qb,
 }
 
 #define MA_TK 64        // keys a tile: one a lane where a wave takes a head's scores
-#define MA_THREADS 256
-#define MA_WAVES 4
+#define MA_THREADS 512   // eight waves: two a SIMD, so that LDS and lane-swap latencies of one hide behind the other
+#define MA_WAVES 8
 
 // eight consecutive elements as floats
 __device__ __forceinline__ void ma_load8(const float* p, float* f) {
@@ -89,13 +90,61 @@ __device__ __forceinline__ void ma_load8(const bf16_t* p, float* f) {
     for (int i = 0; i < 8; ++i) f[i] = (float)pk.h[i];
 }
 
+// A token's visible keys lie in two ranges: the first tokens that are kept (those that the window does not
+// hold anyway), [0, a_hi), and the window, [lo, pos].  Their tiles are numbered through: first those of
+// the first range, then those of the second, each starting at a multiple of MA_TK.
+struct MaTiles {
+    int a_hi, lo, hi, n_a, jt_b, n;
+    __device__ MaTiles(int pos, int window, int keep_first) {
+        lo = window > 0 ? max(0, pos - window + 1) : 0;
+        a_hi = min(keep_first, lo);
+        hi = pos + 1;
+        n_a = (a_hi + MA_TK - 1) / MA_TK;
+        jt_b = (lo / MA_TK) * MA_TK;
+        n = n_a + (pos - jt_b) / MA_TK + 1;
+    }
+};
+
+// One block per (token, split of the token's tiles).  With one split the block writes the token's result;
+// with more it leaves, per head, its running maximum, its sum and the unnormalised weighted values for
+// mixed_attention_merge_kernel (the sink's term is then the merge's to add).
+// Eight consecutive elements as they come from memory; several are asked for before the first is used, so that
+// a thread waits for memory once per group and not once per load.
+template <typename TC> struct MaRaw;
+template <> struct MaRaw<bf16_t> {
+    uint4 u;
+    __device__ __forceinline__ void load(const bf16_t* p) { u = *reinterpret_cast<const uint4*>(p); }
+    __device__ __forceinline__ void zero() { u = make_uint4(0, 0, 0, 0); }
+    __device__ __forceinline__ void get(float* f) const {
+        union { uint4 u; bf16_t h[8]; } pk;
+        pk.u = u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)pk.h[i];
+    }
+};
+template <> struct MaRaw<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float* p) {
+        a = *reinterpret_cast<const float4*>(p);
+        b = *reinterpret_cast<const float4*>(p + 4);
+    }
+    __device__ __forceinline__ void zero() { a = make_float4(0, 0, 0, 0); b = a; }
+    __device__ __forceinline__ void get(float* f) const {
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    }
+};
+
+#define MA_AHEAD 4      // key rows a wave asks for before it multiplies the first
+#define MA_RUNS 4       // runs of 8 values a thread asks for before it multiplies the first
+
 template <typename TC, int ACC>
 __global__ __launch_bounds__(MA_THREADS) void mixed_attention_kernel(
     const TC* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int bt_width, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ positions, const float* __restrict__ bias, int bias_rows,
     const float* __restrict__ mix, float scale, float cap, int window, int keep_first, int sink,
-    TC* __restrict__ out, int H, int G, int D, int page_size) {
+    TC* __restrict__ out, int H, int G, int D, int page_size, int tiles_per_split, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
     extern __shared__ float lds[];
     float* q_s = lds;                       // [H][D]
     float* s_raw = q_s + H * D;             // [H][TK]
@@ -104,173 +153,292 @@ __global__ __launch_bounds__(MA_THREADS) void mixed_attention_kernel(
     float* m_s = mix_s + (mix ? H * H : 0); // [H]
     float* l_s = m_s + H;
     float* c_s = l_s + H;
-    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    // per run of 8 keys of a tile: its page and its place in the page; two sets, by the tile's parity (a wave may
+    // be at the next tile's products while another still weighs this tile's values)
+    int* chunk_s = reinterpret_cast<int*>(c_s + H);      // [2][2][TK / 8]
+    const int t = blockIdx.x, split = blockIdx.y, nsplit = gridDim.y;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int pos = positions[t];
     const int32_t* table = block_tables + (size_t)token_req[t] * bt_width;
     const int rep = H / G, HD = H * D;
-    const bool vec = (D % 8) == 0;
+    const bool own_sink = sink && nsplit == 1;
     for (int i = tid; i < HD; i += MA_THREADS) q_s[i] = to_f32(q[(size_t)t * HD + i]);
     if (mix)
         for (int i = tid; i < H * H; i += MA_THREADS) mix_s[i] = mix[i];
     for (int i = tid; i < H; i += MA_THREADS) {
-        m_s[i] = sink ? 0.f : -INFINITY;
-        l_s[i] = sink ? 1.f : 0.f;
+        m_s[i] = own_sink ? 0.f : -INFINITY;
+        l_s[i] = own_sink ? 1.f : 0.f;
     }
     float acc[ACC];
 #pragma unroll
     for (int n = 0; n < ACC; ++n) acc[n] = 0.f;
     __syncthreads();
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    // two ranges of keys: the first tokens that are kept (those the window does not hold anyway), and the window
-    for (int range = 0; range < 2; ++range) {
-        const int r_lo = range == 0 ? 0 : lo;
-        const int r_hi = range == 0 ? min(keep_first, lo) : pos + 1;     // (exclusive)
-        for (int jt = (r_lo / MA_TK) * MA_TK; jt < r_hi; jt += MA_TK) {
-            // scores of all heads for the tile's keys
-            {
-                const int j = jt + lane;
-                const bool vis = j >= r_lo && j < r_hi;
-                if (vis) {
-                    const int page = table[j / page_size], off = j % page_size;
-                    const int dist = min(pos - j, bias_rows - 1);
-                    for (int g = wv; g < H; g += MA_WAVES) {
-                        const TC* kr = k_cache + (((size_t)page * G + g / rep) * page_size + off) * D;
-                        const float* qg = q_s + g * D;
-                        float dot = 0.f;
-                        if (vec) {
-                            for (int d = 0; d < D; d += 8) {
-                                float kf[8];
-                                ma_load8(kr + d, kf);
-#pragma unroll
-                                for (int e = 0; e < 8; ++e) dot = fmaf(qg[d + e], kf[e], dot);
-                            }
-                        } else {
-                            for (int d = 0; d < D; ++d) dot = fmaf(qg[d], to_f32(kr[d]), dot);
-                        }
-                        float sc = dot * scale;
-                        if (cap > 0.f) sc = cap * tanhf(sc / cap);
-                        if (bias) sc += bias[(size_t)dist * H + g];
-                        s_raw[g * MA_TK + lane] = sc;
-                    }
-                } else {
-                    for (int g = wv; g < H; g += MA_WAVES) s_raw[g * MA_TK + lane] = 0.f;
-                }
-            }
-            __syncthreads();
-            // the heads' scores mixed; the running maximum and sum of each head, a wave a head
-            {
-                const int j = jt + lane;
-                const bool vis = j >= r_lo && j < r_hi;
-                for (int h = wv; h < H; h += MA_WAVES) {
-                    float sc;
-                    if (mix) {
-                        sc = 0.f;
-                        for (int g = 0; g < H; ++g) sc = fmaf(mix_s[h * H + g], s_raw[g * MA_TK + lane], sc);
-                    } else {
-                        sc = s_raw[h * MA_TK + lane];
-                    }
-                    if (!vis) sc = -INFINITY;
-                    const float m_old = m_s[h];
-                    const float m_new = fmaxf(m_old, wave_max(sc));
-                    float p = 0.f, corr = 1.f;
-                    if (m_new > -INFINITY) {
-                        p = vis ? expf(sc - m_new) : 0.f;
-                        corr = expf(m_old - m_new);
-                    }
-                    const float l_new = l_s[h] * corr + wave_sum(p);
-                    p_s[h * MA_TK + lane] = p;
-                    if (lane == 0) {
-                        m_s[h] = m_new;
-                        l_s[h] = l_new;
-                        c_s[h] = corr;
-                    }
-                }
-            }
-            __syncthreads();
-            // weighted values: thread -> (head, element) pairs
-            {
-                const int j_lo = max(jt, r_lo) & ~7, j_hi = min(jt + MA_TK, r_hi);
-#pragma unroll
-                for (int n = 0; n < ACC; ++n) {
-                    const int idx = tid + n * MA_THREADS;
-                    if (idx < HD) {
-                        const int h = idx / D, e = idx % D;
-                        float a = acc[n] * c_s[h];
-                        const float* ph = p_s + h * MA_TK - jt;
-                        for (int j = j_lo; j < j_hi; j += 8) {     // (pages hold a multiple of 8 tokens)
-                            const int page = table[j / page_size], off = j % page_size;
-                            const TC* vr = v_cache + (((size_t)page * G + h / rep) * D + e) * page_size + off;
-                            float vf[8];
-                            ma_load8(vr, vf);
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) a = fmaf(ph[j + i], vf[i], a);
-                        }
-                        acc[n] = a;
-                    }
-                }
-            }
-            // (the next tile's scores go to s_raw, which nobody reads any more; its barrier stands
-            // between these reads of p_s and the next writes)
+    const MaTiles tiles(pos, window, keep_first);
+    const int i_lo = nsplit == 1 ? 0 : split * tiles_per_split;
+    const int i_hi = nsplit == 1 ? tiles.n : min(tiles.n, i_lo + tiles_per_split);
+    // lanes of a key: a key's row of D elements is read by D / 8 neighbouring lanes, 16 bytes each (where D / 8
+    // is a power of two up to 64), so that a wave's load covers whole rows; else a lane reads a key's whole row
+    const int lpk = D / 8;
+    const bool rows_by_lanes = D % 8 == 0 && lpk <= 64 && (lpk & (lpk - 1)) == 0;
+    const int lpk_shift = 31 - __clz(max(lpk, 1));
+    const size_t page_elems = (size_t)G * D * page_size;
+    for (int ti = i_lo; ti < i_hi; ++ti) {
+        const bool first = ti < tiles.n_a;
+        const int jt = first ? ti * MA_TK : tiles.jt_b + (ti - tiles.n_a) * MA_TK;
+        const int r_lo = first ? 0 : tiles.lo, r_hi = first ? tiles.a_hi : tiles.hi;
+        int* chunk = chunk_s + (ti & 1) * (MA_TK / 4);
+        if (tid < MA_TK / 8) {
+            const int j = jt + tid * 8;
+            chunk[tid] = j < r_hi ? table[j / page_size] : 0;       // (no page is looked up past the token's own)
+            chunk[MA_TK / 8 + tid] = j % page_size;
         }
+        // products of all heads' queries with the tile's keys
+        if (rows_by_lanes) {
+            const int kpi = 64 >> lpk_shift;           // keys a wave takes at a time
+            const int kl = lane >> lpk_shift, dl = lane & (lpk - 1);
+            const int its = G << lpk_shift;            // (MA_TK / kpi = lpk rounds a kv head)
+            for (int it0 = wv; it0 < its; it0 += MA_WAVES * MA_AHEAD) {
+                MaRaw<TC> rows[MA_AHEAD];
+#pragma unroll
+                for (int a = 0; a < MA_AHEAD; ++a) {
+                    const int it = it0 + a * MA_WAVES;
+                    const int kvh = it >> lpk_shift, j = jt + (it & (lpk - 1)) * kpi + kl;
+                    rows[a].zero();
+                    if (it < its && j >= r_lo && j < r_hi) {
+                        const int page = table[j / page_size], off = j % page_size;
+                        rows[a].load(k_cache + (((size_t)page * G + kvh) * page_size + off) * D + dl * 8);
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < MA_AHEAD; ++a) {
+                    const int it = it0 + a * MA_WAVES;
+                    if (it >= its) break;
+                    const int kvh = it >> lpk_shift, key = (it & (lpk - 1)) * kpi + kl;
+                    float kf[8];
+                    rows[a].get(kf);
+                    for (int g = kvh * rep; g < (kvh + 1) * rep; ++g) {
+                        const float4* q4 = reinterpret_cast<const float4*>(q_s + g * D + dl * 8);
+                        const float4 qa = q4[0], qb = q4[1];
+                        float dot = qa.x * kf[0];
+                        dot = fmaf(qa.y, kf[1], dot); dot = fmaf(qa.z, kf[2], dot); dot = fmaf(qa.w, kf[3], dot);
+                        dot = fmaf(qb.x, kf[4], dot); dot = fmaf(qb.y, kf[5], dot); dot = fmaf(qb.z, kf[6], dot);
+                        dot = fmaf(qb.w, kf[7], dot);
+                        for (int o = 1; o < lpk; o <<= 1) dot += __shfl_xor(dot, o, 64);
+                        if (dl == 0) s_raw[g * MA_TK + key] = dot;
+                    }
+                }
+            }
+        } else {
+            const int j = jt + lane;
+            const bool vis = j >= r_lo && j < r_hi;
+            if (vis) {
+                const int page = table[j / page_size], off = j % page_size;
+                for (int g = wv; g < H; g += MA_WAVES) {
+                    const TC* kr = k_cache + (((size_t)page * G + g / rep) * page_size + off) * D;
+                    const float* qg = q_s + g * D;
+                    float dot = 0.f;
+                    for (int d = 0; d < D; ++d) dot = fmaf(qg[d], to_f32(kr[d]), dot);
+                    s_raw[g * MA_TK + lane] = dot;
+                }
+            } else {
+                for (int g = wv; g < H; g += MA_WAVES) s_raw[g * MA_TK + lane] = 0.f;
+            }
+        }
+        __syncthreads();
+        // scale, soft cap and the bias of the distance: a lane a key, a wave a head at a time
+        {
+            const int j = jt + lane;
+            const bool vis = j >= r_lo && j < r_hi;
+            const int dist = min(pos - j, bias_rows - 1);
+            for (int g = wv; g < H; g += MA_WAVES) {
+                float sc = 0.f;
+                if (vis) {
+                    sc = s_raw[g * MA_TK + lane] * scale;
+                    if (cap > 0.f) sc = cap * tanhf(sc / cap);
+                    if (bias) sc += bias[(size_t)dist * H + g];
+                }
+                s_raw[g * MA_TK + lane] = sc;
+            }
+        }
+        __syncthreads();
+        // the heads' scores mixed; the running maximum and sum of each head, a wave a head
+        {
+            const int j = jt + lane;
+            const bool vis = j >= r_lo && j < r_hi;
+            for (int h = wv; h < H; h += MA_WAVES) {
+                float sc;
+                if (mix) {
+                    sc = 0.f;
+                    for (int g = 0; g < H; ++g) sc = fmaf(mix_s[h * H + g], s_raw[g * MA_TK + lane], sc);
+                } else {
+                    sc = s_raw[h * MA_TK + lane];
+                }
+                if (!vis) sc = -INFINITY;
+                const float m_old = m_s[h];
+                const float m_new = fmaxf(m_old, wave_max(sc));
+                float p = 0.f, corr = 1.f;
+                if (m_new > -INFINITY) {
+                    p = vis ? expf(sc - m_new) : 0.f;
+                    corr = expf(m_old - m_new);
+                }
+                const float l_new = l_s[h] * corr + wave_sum(p);
+                p_s[h * MA_TK + lane] = p;
+                if (lane == 0) {
+                    m_s[h] = m_new;
+                    l_s[h] = l_new;
+                    c_s[h] = corr;
+                }
+            }
+        }
+        __syncthreads();
+        // weighted values: thread -> (head, element) pairs; the tile's runs of 8 keys are asked for four at a time
+        {
+            const int c_lo = (max(jt, r_lo) - jt) >> 3, c_hi = (min(jt + MA_TK, r_hi) - jt + 7) >> 3;
+#pragma unroll
+            for (int n = 0; n < ACC; ++n) {
+                const int idx = tid + n * MA_THREADS;
+                if (idx < HD) {
+                    const int h = idx / D;
+                    const int voff = ((h / rep) * D + idx % D) * page_size;      // (kv head, element) in a value page
+                    float a = acc[n] * c_s[h];
+                    const float* ph = p_s + h * MA_TK;
+#pragma unroll
+                    for (int c0 = 0; c0 < MA_TK / 8; c0 += MA_RUNS) {
+                        MaRaw<TC> runs[MA_RUNS];
+#pragma unroll
+                        for (int c = 0; c < MA_RUNS; ++c) {
+                            runs[c].zero();
+                            if (c0 + c >= c_lo && c0 + c < c_hi)        // (pages hold a multiple of 8 tokens)
+                                runs[c].load(v_cache + (size_t)chunk[c0 + c] * page_elems + chunk[MA_TK / 8 + c0 + c] + voff);
+                        }
+#pragma unroll
+                        for (int c = 0; c < MA_RUNS; ++c) {
+                            float vf[8];
+                            runs[c].get(vf);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) a = fmaf(ph[(c0 + c) * 8 + i], vf[i], a);
+                        }
+                    }
+                    acc[n] = a;
+                }
+            }
+        }
+        // (the next tile's scores go to s_raw, which nobody reads any more; its barrier stands
+        // between these reads of p_s and the next writes)
     }
     __syncthreads();
+    if (nsplit == 1) {
+#pragma unroll
+        for (int n = 0; n < ACC; ++n) {
+            const int idx = tid + n * MA_THREADS;
+            if (idx < HD) {
+                const float l = l_s[idx / D];
+                out[(size_t)t * HD + idx] = from_f32<TC>(l > 0.f ? acc[n] / l : 0.f);
+            }
+        }
+        return;
+    }
+    float* po = part_o + ((size_t)t * nsplit + split) * HD;
 #pragma unroll
     for (int n = 0; n < ACC; ++n) {
         const int idx = tid + n * MA_THREADS;
-        if (idx < HD) {
-            const float l = l_s[idx / D];
-            out[(size_t)t * HD + idx] = from_f32<TC>(l > 0.f ? acc[n] / l : 0.f);
+        if (idx < HD) po[idx] = acc[n];
+    }
+    float* pm = part_ml + ((size_t)t * nsplit + split) * 2 * H;
+    for (int i = tid; i < H; i += MA_THREADS) {
+        pm[i] = m_s[i];
+        pm[H + i] = l_s[i];
+    }
+}
+
+// The splits of a token's keys put together, in the order of the splits: M = max of the maxima (and 0, the
+// sink's score), L = [sink] e^-M + sum_s l_s e^(m_s - M), out = sum_s o_s e^(m_s - M) / L.
+template <typename TC>
+__global__ __launch_bounds__(64) void mixed_attention_merge_kernel(const float* __restrict__ part_o,
+                                                                   const float* __restrict__ part_ml, int nsplit,
+                                                                   int sink, TC* __restrict__ out, int H, int D) {
+    const int t = blockIdx.x / H, h = blockIdx.x % H, HD = H * D;
+    const float* pm = part_ml + (size_t)t * nsplit * 2 * H;
+    const float* po = part_o + (size_t)t * nsplit * HD + (size_t)h * D;
+    float M = sink ? 0.f : -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pm[s * 2 * H + h]);
+    float L = sink ? expf(-M) : 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float m = pm[s * 2 * H + h];
+        if (m > -INFINITY) L = fmaf(pm[s * 2 * H + H + h], expf(m - M), L);
+    }
+    for (int e = threadIdx.x; e < D; e += 64) {
+        float a = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float m = pm[s * 2 * H + h];
+            if (m > -INFINITY) a = fmaf(po[(size_t)s * HD + e], expf(m - M), a);
         }
+        out[(size_t)t * HD + (size_t)h * D + e] = from_f32<TC>(L > 0.f ? a / L : 0.f);
     }
 }
 
 static size_t ma_lds_bytes(int H, int D, bool mix) {
-    return sizeof(float) * ((size_t)H * D + 2 * (size_t)H * MA_TK + (mix ? (size_t)H * H : 0) + 3 * (size_t)H);
+    return sizeof(float) * ((size_t)H * D + 2 * (size_t)H * MA_TK + (mix ? (size_t)H * H : 0) + 3 * (size_t)H + MA_TK / 2);
 }
 
 TFF_API int tff_mixed_attention_supported(int H, int D, int has_mix) {
-    return H > 0 && D > 0 && (size_t)H * D <= 16 * MA_THREADS && ma_lds_bytes(H, D, has_mix != 0) <= 64 * 1024;
+    return H > 0 && D > 0 && (size_t)H * D <= 8 * MA_THREADS && ma_lds_bytes(H, D, has_mix != 0) <= 64 * 1024;
+}
+
+// Floats of workspace that `splits` splits of T tokens need (0 for one split).
+TFF_API size_t tff_mixed_attention_workspace_bytes(int T, int H, int D, int splits) {
+    return splits <= 1 ? 0 : sizeof(float) * (size_t)T * splits * ((size_t)H * D + 2 * (size_t)H);
 }
 
 template <typename TC>
 static int ma_launch(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, int bt_width,
                      const int32_t* token_req, const int32_t* positions, const float* bias, int bias_rows, const float* mix,
                      float scale, float cap, int window, int keep_first, int sink, void* out, int T, int H, int G, int D,
-                     int page_size, hipStream_t s) {
+                     int page_size, int splits, int tiles_per_split, float* ws, hipStream_t s) {
     const size_t lds = ma_lds_bytes(H, D, mix != nullptr);
     const int per = (H * D + MA_THREADS - 1) / MA_THREADS;
+    float* part_o = ws;
+    float* part_ml = ws ? ws + (size_t)T * splits * H * D : nullptr;
+    const dim3 grid(T, splits);
 #define MA_LAUNCH(ACC)                                                                                                   \
-    mixed_attention_kernel<TC, ACC><<<T, MA_THREADS, lds, s>>>((const TC*)q, (const TC*)k_cache, (const TC*)v_cache,      \
-                                                                block_tables, bt_width, token_req, positions, bias,      \
-                                                                bias_rows, mix, scale, cap, window, keep_first, sink,    \
-                                                                (TC*)out, H, G, D, page_size)
+    mixed_attention_kernel<TC, ACC><<<grid, MA_THREADS, lds, s>>>((const TC*)q, (const TC*)k_cache, (const TC*)v_cache,   \
+                                                                   block_tables, bt_width, token_req, positions, bias,   \
+                                                                   bias_rows, mix, scale, cap, window, keep_first, sink, \
+                                                                   (TC*)out, H, G, D, page_size, tiles_per_split, part_o, \
+                                                                   part_ml)
     if (per <= 1) MA_LAUNCH(1);
     else if (per <= 2) MA_LAUNCH(2);
     else if (per <= 4) MA_LAUNCH(4);
-    else if (per <= 8) MA_LAUNCH(8);
-    else MA_LAUNCH(16);
+    else MA_LAUNCH(8);
 #undef MA_LAUNCH
-    return tff_check_launch("mixed_attention");
+    int rc = tff_check_launch("mixed_attention");
+    if (rc || splits <= 1) return rc;
+    mixed_attention_merge_kernel<TC><<<T * H, 64, 0, s>>>(part_o, part_ml, splits, sink, (TC*)out, H, D);
+    return tff_check_launch("mixed_attention_merge");
 }
 
 TFF_API int tff_mixed_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                 int bt_width, const int32_t* token_req, const int32_t* positions, const float* bias,
                                 int bias_rows, const float* mix, float scale, float cap, int window, int keep_first,
-                                int sink, void* out, int T, int H, int G, int D, int page_size, int dtype,
-                                tff_stream_t stream) {
+                                int sink, void* out, int T, int H, int G, int D, int page_size, int splits,
+                                int tiles_per_split, float* workspace, int dtype, tff_stream_t stream) {
     TFF_REQUIRE(q && k_cache && v_cache && block_tables && token_req && positions && out, "mixed_attention: null pointer");
     TFF_REQUIRE(T >= 0 && G > 0 && H % G == 0 && bt_width > 0 && page_size > 0 && page_size % 8 == 0,
                 "mixed_attention: %d heads on %d kv heads, pages of %d", H, G, page_size);
     TFF_REQUIRE(tff_mixed_attention_supported(H, D, mix != nullptr), "mixed_attention: %d heads of %d do not fit a block", H, D);
     TFF_REQUIRE(!bias || bias_rows > 0, "mixed_attention: a bias table without rows");
     TFF_REQUIRE(window >= 0 && keep_first >= 0, "mixed_attention: negative window");
+    TFF_REQUIRE(splits >= 1 && splits <= 65535 && (splits == 1 || (tiles_per_split >= 1 && workspace)),
+                "mixed_attention: %d splits of %d tiles", splits, tiles_per_split);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TFF_F32)
         return ma_launch<float>(q, k_cache, v_cache, block_tables, bt_width, token_req, positions, bias, bias_rows, mix,
-                                scale, cap, window, keep_first, sink, out, T, H, G, D, page_size, s);
+                                scale, cap, window, keep_first, sink, out, T, H, G, D, page_size, splits, tiles_per_split,
+                                workspace, s);
     if (dtype == TFF_BF16)
         return ma_launch<bf16_t>(q, k_cache, v_cache, block_tables, bt_width, token_req, positions, bias, bias_rows, mix,
-                                 scale, cap, window, keep_first, sink, out, T, H, G, D, page_size, s);
+                                 scale, cap, window, keep_first, sink, out, T, H, G, D, page_size, splits, tiles_per_split,
+                                 workspace, s);
     return tff_fail("mixed_attention: unknown dtype %d", dtype);
 }

@@ -320,8 +320,11 @@ TFF_API int tff_mixed_attention_supported(int H, int D, int has_mix);
 TFF_API int tff_mixed_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                 int bt_width, const int32_t* token_req, const int32_t* positions, const float* bias,
                                 int bias_rows, const float* mix, float scale, float cap, int window, int keep_first,
-                                int sink, void* out, int T, int H, int G, int D, int page_size, int dtype,
-                                tff_stream_t stream);
+                                int sink, void* out, int T, int H, int G, int D, int page_size, int splits,
+                                int tiles_per_split, float* workspace, int dtype, tff_stream_t stream);
+// splits > 1: each token's tiles of 64 keys are dealt to `splits` blocks, tiles_per_split each, and merged by a
+// second kernel; workspace of tff_mixed_attention_workspace_bytes(T, H, D, splits) bytes.
+TFF_API size_t tff_mixed_attention_workspace_bytes(int T, int H, int D, int splits);
 
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

@@ -30,7 +30,8 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(
     const float* prev = (t == cu_tokens[r]) ? state + (size_t)state_slots[r] * state_row + prev_off
                                             : x + (size_t)(t - 1) * W;
     const float* xr = x + (size_t)t * W;
-    for (int c = threadIdx.x; c < W; c += 256) {
+    const int c = blockIdx.y * 256 + threadIdx.x;      // (a block a token and 256 columns: few tokens still fill the GPU)
+    if (c < W) {
         const float h = xr[c];
         const float d = prev[c] - h;
         for (int m = 0; m < M; ++m) out[((size_t)m * T + t) * W + c] = from_f32<TO>(h + d * mu[(size_t)m * W + c]);
@@ -44,11 +45,12 @@ TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state
     TFF_REQUIRE(T >= 0 && W > 0 && M > 0 && prev_off + (size_t)W <= state_row, "token_shift_mix: bad sizes");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T, (W + 255) / 256);
     if (out_dtype == TFF_F32)
-        token_shift_mix_kernel<float><<<T, 256, 0, s>>>(x, state, state_row, prev_off, mu, M, token_req, cu_tokens,
+        token_shift_mix_kernel<float><<<grid, 256, 0, s>>>(x, state, state_row, prev_off, mu, M, token_req, cu_tokens,
                                                          state_slots, (float*)out, T, W);
     else if (out_dtype == TFF_BF16)
-        token_shift_mix_kernel<bf16_t><<<T, 256, 0, s>>>(x, state, state_row, prev_off, mu, M, token_req, cu_tokens,
+        token_shift_mix_kernel<bf16_t><<<grid, 256, 0, s>>>(x, state, state_row, prev_off, mu, M, token_req, cu_tokens,
                                                           state_slots, (bf16_t*)out, T, W);
     else
         return tff_fail("token_shift_mix: unknown dtype %d", out_dtype);
@@ -57,13 +59,15 @@ TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state
 
 #define WKV_MAX_D 128     // (a thread keeps a slice of a column of S in registers)
 #define WKV_MAX_SLICES 4
-#define WKV_CHUNK_ELEMS 1024   // tokens of a chunk x head size, at most
+#define WKV_CHUNK_ELEMS 1024   // tokens of a chunk x padded head size, at most
 #define WKV_EPT 4              // elements of a chunk's array a thread fetches, at most
 
 // KPT key channels a thread; ceil(D / KPT) <= 4 slices of the key channels; thread = slice * D + value channel.
 // The tokens of a portion pass in chunks of up to 16: a chunk's r, k, w, v are fetched into registers while the
 // chunk before it is worked through from LDS, so that no token waits for memory; within a chunk a token costs
-// its multiply-adds and one barrier (the slices' partial sums meet in LDS, in a buffer of the token's parity).
+// its multiply-adds, its slice of r, k, w in 16-byte LDS reads and one barrier (the slices' partial sums meet
+// in LDS, in a buffer of the token's parity).  In LDS a token's channels lie Dp = slices * KPT apart, the
+// channels past D zero, so that a slice needs no bounds.
 template <int KPT>
 __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
@@ -71,26 +75,28 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     float* __restrict__ state, size_t state_row, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ state_slots, float* __restrict__ o, int H, int D, const float* __restrict__ x, int W,
     size_t prev_off) {
-    __shared__ float buf[2][4][WKV_CHUNK_ELEMS];       // r, k, w, v of a chunk, [token in chunk][channel]
+    __shared__ __attribute__((aligned(16))) float buf[2][3][WKV_CHUNK_ELEMS];       // r, k, w of a chunk, [token][channel]
+    __shared__ float bv[2][WKV_CHUNK_ELEMS];                                       // v of a chunk
     __shared__ float so[WKV_CHUNK_ELEMS];
-    __shared__ float su[WKV_MAX_D];
     __shared__ float part[2][WKV_MAX_SLICES][WKV_MAX_D];
     const int h = blockIdx.x, req = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
     const int t0 = cu_tokens[req], t1 = cu_tokens[req + 1];
     if (t1 <= t0) return;
     const int slices = nt / D;
+    const int Dp = slices * KPT;
     const int vi = tid % D, ks = tid / D;
-    const int C = min(min(16, WKV_EPT * slices), WKV_CHUNK_ELEMS / D);      // tokens a chunk
+    const int C = min(min(16, WKV_EPT * slices), WKV_CHUNK_ELEMS / Dp);      // tokens a chunk
     float* srow = state + (size_t)state_slots[req] * state_row;
     float* S = srow + (size_t)h * D * D;
     const size_t col = (size_t)h * D;
-    float s[KPT];
+    float s[KPT], uu[KPT];
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
         const int kk = ks * KPT + i;
         s[i] = kk < D ? S[(size_t)kk * D + vi] : 0.f;
+        uu[i] = kk < D ? u[col + kk] : 0.f;
     }
-    if (tid < D) su[tid] = u[col + tid];
+    for (int e = tid; e < 2 * 3 * WKV_CHUNK_ELEMS; e += nt) (&buf[0][0][0])[e] = 0.f;      // (the channels past D stay zero)
     float fr[WKV_EPT], fk[WKV_EPT], fz[WKV_EPT], fv[WKV_EPT];
     // a chunk's elements e = token * D + channel are dealt to the threads in strides of the block
     auto fetch = [&](int base) {
@@ -113,14 +119,16 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
         for (int i = 0; i < WKV_EPT; ++i) {
             const int e = tid + i * nt;
             if (e < n) {
-                buf[b][0][e] = fr[i];
-                buf[b][1][e] = fk[i];
-                buf[b][2][e] = expf(-expf(fz[i]));
-                buf[b][3][e] = fv[i];
+                const int at = (e / D) * Dp + e % D;
+                buf[b][0][at] = fr[i];
+                buf[b][1][at] = fk[i];
+                buf[b][2][at] = expf(-expf(fz[i]));
+                bv[b][e] = fv[i];
             }
         }
     };
     fetch(t0);
+    __syncthreads();
     stage(t0, 0);
     int b = 0;
     for (int base = t0; base < t1; base += C, b ^= 1) {
@@ -128,18 +136,21 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
         __syncthreads();
         if (base + C < t1) fetch(base + C);
         for (int c = 0; c < n; ++c) {
-            const float* cr = buf[b][0] + c * D;
-            const float* ck = buf[b][1] + c * D;
-            const float* cw = buf[b][2] + c * D;
-            const float vt = buf[b][3][c * D + vi];
+            const float4* cr = reinterpret_cast<const float4*>(buf[b][0] + c * Dp + ks * KPT);
+            const float4* ck = reinterpret_cast<const float4*>(buf[b][1] + c * Dp + ks * KPT);
+            const float4* cw = reinterpret_cast<const float4*>(buf[b][2] + c * Dp + ks * KPT);
+            const float vt = bv[b][c * D + vi];
             float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < KPT; ++i) {
-                const int kk = ks * KPT + i;
-                if (kk < D) {
-                    const float kv = ck[kk] * vt;
-                    acc = fmaf(cr[kk], fmaf(su[kk], kv, s[i]), acc);
-                    s[i] = fmaf(cw[kk], s[i], kv);
+            for (int i = 0; i < KPT; i += 4) {
+                const float4 r4 = cr[i >> 2], k4 = ck[i >> 2], w4 = cw[i >> 2];
+                const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk4[4] = {k4.x, k4.y, k4.z, k4.w},
+                            ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float kv = kk4[j] * vt;
+                    acc = fmaf(rr[j], fmaf(uu[i + j], kv, s[i + j]), acc);
+                    s[i + j] = fmaf(ww[j], s[i + j], kv);
                 }
             }
             part[c & 1][ks][vi] = acc;
@@ -165,6 +176,103 @@ __global__ __launch_bounds__(512) void wkv_recurrence_kernel(
     }
 }
 
+// The same for head sizes that are multiples of 16 (D = 4 * KPT): a wave takes sixteen value channels, its four
+// rows of sixteen lanes a quarter of the key channels each, and the quarters' partial sums meet through lane
+// swaps: no barrier and no LDS between the tokens of a chunk, the waves run on their own.
+template <int KPT>
+__global__ __launch_bounds__(512) void wkv_recurrence_wave_kernel(
+    const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
+    const float* __restrict__ z, size_t row, const float* __restrict__ w0, const float* __restrict__ u,
+    float* __restrict__ state, size_t state_row, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ state_slots, float* __restrict__ o, int H, const float* __restrict__ x, int W,
+    size_t prev_off) {
+    constexpr int D = 4 * KPT;
+    constexpr int C = (WKV_CHUNK_ELEMS / D) < 16 ? (WKV_CHUNK_ELEMS / D) : 16;      // tokens a chunk
+    constexpr int NT = 4 * D;                                                      // threads: D / 16 waves
+    constexpr int EPT = (C * D + NT - 1) / NT;
+    __shared__ __attribute__((aligned(16))) float buf[2][3][C * D];       // r, k, w of a chunk, [token][channel]
+    __shared__ float bv[2][C * D];
+    const int h = blockIdx.x, req = blockIdx.y, tid = threadIdx.x;
+    const int t0 = cu_tokens[req], t1 = cu_tokens[req + 1];
+    if (t1 <= t0) return;
+    const int lane = tid & 63;
+    const int ks = lane >> 4, vi = (tid >> 6) * 16 + (lane & 15);
+    float* srow = state + (size_t)state_slots[req] * state_row;
+    float* S = srow + (size_t)h * D * D;
+    const size_t col = (size_t)h * D;
+    float s[KPT], uu[KPT];
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+        s[i] = S[(size_t)(ks * KPT + i) * D + vi];
+        uu[i] = u[col + ks * KPT + i];
+    }
+    float fr[EPT], fk[EPT], fz[EPT], fv[EPT];
+    auto fetch = [&](int base) {
+        const int n = min(C, t1 - base) * D;
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+            const int e = tid + i * NT;
+            if (e < n) {
+                const size_t a = (size_t)(base + e / D) * row + col + e % D;
+                fr[i] = r[a];
+                fk[i] = k[a];
+                fz[i] = z[a] + w0[col + e % D];
+                fv[i] = v[a];
+            }
+        }
+    };
+    auto stage = [&](int base, int b) {
+        const int n = min(C, t1 - base) * D;
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+            const int e = tid + i * NT;
+            if (e < n) {
+                buf[b][0][e] = fr[i];
+                buf[b][1][e] = fk[i];
+                buf[b][2][e] = expf(-expf(fz[i]));
+                bv[b][e] = fv[i];
+            }
+        }
+    };
+    fetch(t0);
+    stage(t0, 0);
+    int b = 0;
+    for (int base = t0; base < t1; base += C, b ^= 1) {
+        const int n = min(C, t1 - base);
+        __syncthreads();
+        if (base + C < t1) fetch(base + C);
+        for (int c = 0; c < n; ++c) {
+            const float4* cr = reinterpret_cast<const float4*>(buf[b][0] + c * D + ks * KPT);
+            const float4* ck = reinterpret_cast<const float4*>(buf[b][1] + c * D + ks * KPT);
+            const float4* cw = reinterpret_cast<const float4*>(buf[b][2] + c * D + ks * KPT);
+            const float vt = bv[b][c * D + vi];
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < KPT; i += 4) {
+                const float4 r4 = cr[i >> 2], k4 = ck[i >> 2], w4 = cw[i >> 2];
+                const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk4[4] = {k4.x, k4.y, k4.z, k4.w},
+                            ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float kv = kk4[j] * vt;
+                    acc = fmaf(rr[j], fmaf(uu[i + j], kv, s[i + j]), acc);
+                    s[i + j] = fmaf(ww[j], s[i + j], kv);
+                }
+            }
+            acc = rows_sum(acc);        // (quarter 0 + quarter 1) + (quarter 2 + quarter 3), in every lane
+            if (ks == 0) o[(size_t)(base + c) * H * D + col + vi] = acc;
+        }
+        // (the other buffer was last read before this round's barrier)
+        if (base + C < t1) stage(base + C, b ^ 1);
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) S[(size_t)(ks * KPT + i) * D + vi] = s[i];
+    if (h == 0 && x) {
+        const float* last = x + (size_t)(t1 - 1) * W;
+        for (int c = tid; c < W; c += NT) srow[prev_off + c] = last[c];
+    }
+}
+
 TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, const float* z, size_t row, const float* w0,
                                const float* u, float* state, size_t state_row, const int32_t* cu_tokens,
                                const int32_t* state_slots, float* o, int R, int H, int D, const float* x, int W,
@@ -179,8 +287,23 @@ TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, c
 #define WKV_LAUNCH(KPT)                                                                                              \
     wkv_recurrence_kernel<KPT><<<grid, D * ((D + KPT - 1) / KPT), 0, s>>>(r, k, v, z, row, w0, u, state, state_row, \
                                                                            cu_tokens, state_slots, o, H, D, x, W, prev_off)
-    if (D <= 64) WKV_LAUNCH(16);
+#define WKV_WAVES(KPT)                                                                                             \
+    wkv_recurrence_wave_kernel<KPT><<<grid, 16 * KPT, 0, s>>>(r, k, v, z, row, w0, u, state, state_row, cu_tokens, \
+                                                              state_slots, o, H, x, W, prev_off)
+    if (D % 16 == 0) {
+        switch (D / 4) {
+            case 4: WKV_WAVES(4); break;
+            case 8: WKV_WAVES(8); break;
+            case 12: WKV_WAVES(12); break;
+            case 16: WKV_WAVES(16); break;
+            case 20: WKV_WAVES(20); break;
+            case 24: WKV_WAVES(24); break;
+            case 28: WKV_WAVES(28); break;
+            default: WKV_WAVES(32); break;
+        }
+    } else if (D <= 64) WKV_LAUNCH(16);
     else WKV_LAUNCH(32);
+#undef WKV_WAVES
 #undef WKV_LAUNCH
     return tff_check_launch("wkv_recurrence");
 }

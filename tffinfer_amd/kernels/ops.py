@@ -1284,15 +1284,21 @@ def qk_bias_norm_store(qk: torch.Tensor, q_bias, k_bias, eps: float, H: int, G: 
     return q
 
 
+#: blocks a step of few tokens spreads its attention over (two a CU)
+MIXED_ATTENTION_BLOCKS = 512
+
+
 def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: float, softcap: float = 0.0,
                     bias: torch.Tensor | None = None, mix: torch.Tensor | None = None, window: int = 0,
-                    keep_first: int = 0, sink: bool = False) -> torch.Tensor:
+                    keep_first: int = 0, sink: bool = False, splits: int | None = None) -> torch.Tensor:
     """Causal attention over the paged cache whose heads exchange their scores before the softmax:
     s_g = softcap * tanh(scale * q_g . k_g / softcap) (softcap 0: scale * q_g . k_g) + bias[min(i - j, rows - 1), g];
     s'_h = sum_g mix[h, g] s_g; key j is visible to query i if j <= i and (i - j < window or j < keep_first)
     (window 0: all j <= i); softmax over the visible keys, with one more term of 1 in the denominator
     if ``sink``; the values are the value pages.  q [T, H * D] in the cache's type; bias float32 [rows, H];
-    mix float32 [H, H]."""
+    mix float32 [H, H].  A step of few tokens deals each token's keys (tiles of 64) to several blocks
+    (``splits``; by default so many that some 512 blocks run, from the longest context the step's tables
+    can hold) and merges them in a second kernel."""
     dt = kv.k_cache.dtype
     _req(q, "mixed_attention q", dt, 2)
     T = q.shape[0]
@@ -1316,11 +1322,22 @@ def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: f
     if batch.token_req.numel() < T or batch.positions.numel() < T:
         raise _lib.KernelError("mixed_attention: the step's tables are shorter than q")
     out = torch.empty(T, H * D, dtype=dt, device=q.device)
+    # tiles of 64 keys that a token of this step can have at most (what the block tables can hold, or the window
+    # and the kept tokens): a size the host knows without reading a position, so a captured step keeps it
+    reach = bt.shape[1] * kv.page_size
+    tiles = -(-min(keep_first, reach) // 64) + (-(-min(window, reach) // 64) + 1 if window > 0 else -(-reach // 64))
+    if splits is None:
+        splits = max(1, min(tiles, MIXED_ATTENTION_BLOCKS // max(T, 1)))
+    per = -(-tiles // max(1, splits))
+    splits = -(-tiles // per) if splits > 1 else 1
+    ws = None
+    if splits > 1:
+        ws = torch.empty(L.tff_mixed_attention_workspace_bytes(T, H, D, splits) // 4, dtype=torch.float32, device=q.device)
     _lib.check(L.tff_mixed_attention(q.data_ptr(), kv.k_cache.data_ptr(), kv.v_cache.data_ptr(), bt.data_ptr(),
                                      bt.shape[1], batch.token_req.data_ptr(), batch.positions.data_ptr(), _ptr(bias),
                                      rows, _ptr(mix), float(scale), float(softcap), int(window), int(keep_first),
-                                     1 if sink else 0, out.data_ptr(), T, H, G, D, kv.page_size, dtype_code(dt),
-                                     _stream()))
+                                     1 if sink else 0, out.data_ptr(), T, H, G, D, kv.page_size, splits, per, _ptr(ws),
+                                     dtype_code(dt), _stream()))
     return out
 
 
