@@ -40,6 +40,7 @@ def _batch(lengths, starts, slots=None):
         pos += list(range(s, s + n))
         req += [r] * n
     return types.SimpleNamespace(token_req=_i32(req), positions=_i32(pos), cu_tokens=_i32(cu), num_reqs=len(lengths),
+                                 max_new_tokens=max(lengths),
                                  state_slots=_i32(slots if slots is not None else list(range(len(lengths)))))
 
 
@@ -142,7 +143,11 @@ def test_recurrence_whole_and_in_portions(H, D):
                                x=x[idx].to(DEV), prev_off=H * D * D)
         got.append(o[:n])
         at += n
-    assert torch.equal(torch.cat(got, 0), whole)
+    # (heads of 64 and 128 run long portions in a form of their own, whose sums go in another order)
+    if D in (64, 128):
+        assert _err(torch.cat(got, 0), whole) < 2e-6
+    else:
+        assert torch.equal(torch.cat(got, 0), whole)
 
 
 @pytest.mark.parametrize("H,D", [(3, 8), (2, 40), (1, 128)])
@@ -355,12 +360,11 @@ def requests_for(name, model_dir):
 
 
 def check(model_dir, reqs, steps, results, dtype, name):
-    """All rows in float32; in bfloat16 a request's rows before its first close call among the experts."""
-    before = None
-    if dtype == "bfloat16":
-        before = {rid: comparable_tokens(model_dir, tuple(toks)) for rid, toks in reqs.items()}
-        total = sum(len(t) for t in reqs.values())
-        assert sum(before.values()) >= total // 5, "too little of these requests can be compared in bfloat16"
+    """A request's rows before its first close call: in bfloat16 among the experts' scores, in both types a first
+    token whose recurrence output all but cancels."""
+    before = {rid: comparable_tokens(model_dir, tuple(toks), dtype) for rid, toks in reqs.items()}
+    total = sum(len(t) for t in reqs.values())
+    assert sum(before.values()) >= total // (5 if dtype == "bfloat16" else 2), "too little of these requests can be compared"
     return rl.check_against_oracle(model_dir, reqs, steps, results, tol(dtype, name), dtype, compare_before=before)
 
 

@@ -301,10 +301,11 @@ TFF_API int tff_token_shift_mix(const float* x, const float* state, size_t state
 // r, k, v, z float32 [T, >= H * D] with rows `row` elements apart; w = exp(-exp(z + w0)); per request (cu_tokens,
 // state_slots) and head, state[slot, h] = S [D, D]: o_t = (S + diag(u) k v^T)^T r, S <- diag(w) S + k v^T.
 // o float32 [T, H * D].  x (optional) [T, W]: the portion's last row goes to state[slot, prev_off : prev_off + W].
+// long_portions: the step holds prompts' portions (the form whose cost per token is least; heads of 64 and 128).
 TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, const float* z, size_t row, const float* w0,
                                const float* u, float* state, size_t state_row, const int32_t* cu_tokens,
                                const int32_t* state_slots, float* o, int R, int H, int D, const float* x, int W,
-                               size_t prev_off, tff_stream_t stream);
+                               size_t prev_off, int long_portions, tff_stream_t stream);
 // out = o / sqrt(mean over each head of o^2 + eps) * nw * silu(g); g rows g_row elements apart.
 TFF_API int tff_head_norm_gate(const float* o, const float* g, size_t g_row, const float* nw, float eps, void* out, int T,
                                int H, int D, int out_dtype, tff_stream_t stream);

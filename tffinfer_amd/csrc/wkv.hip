@@ -12,8 +12,10 @@
 //   the row that the state keeps (zeros for a request's first token).
 // tff_wkv_recurrence: the recurrence over the tokens of each request's portion, one block per
 //   (head, request), a thread per value channel and slice of the key channels; the order of every
-//   sum is fixed by the head size alone, so a token's result does not depend on how the tokens
-//   were cut into steps.  The block of head 0 also leaves the portion's last row of x in the state.
+//   sum is fixed by the head size and the kernel's form alone, so a token's result does not depend on
+//   how the tokens were cut into steps beyond rounding (`long_portions` picks the form for prompts, whose
+//   sums run in another order than those of the form for single tokens).  The block of head 0 also
+//   leaves the portion's last row of x in the state.
 // tff_head_norm_gate: out = o / sqrt(mean over the head of o^2 + eps) * weight * silu(g).
 // tff_tanh: out = tanh(in), float32 in, the activation type out.
 #include "common.h"
@@ -273,10 +275,141 @@ __global__ __launch_bounds__(512) void wkv_recurrence_wave_kernel(
     }
 }
 
+// Sum over the sixteen lanes of a row, the result in all of them: neighbours, pairs, the two quads of a half,
+// the two halves (data-parallel primitives: no LDS); the order of the additions is fixed.
+__device__ __forceinline__ float row16_sum(float v) {
+#define WKV_DPP(x, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xF, 0xF, true))
+    v += WKV_DPP(v, 0xB1);       // quad_perm [1, 0, 3, 2]
+    v += WKV_DPP(v, 0x4E);       // quad_perm [2, 3, 0, 1]
+    v += WKV_DPP(v, 0x141);      // row_half_mirror
+    v += WKV_DPP(v, 0x140);      // row_mirror
+#undef WKV_DPP
+    return v;
+}
+
+// For long portions (prompts) of heads of 64 or 128 channels (D = 16 * KPT): a token's cost is what bounds a
+// prompt, since its tokens go one after the other.  Here a row of sixteen lanes shares a value channel, each
+// lane KPT key channels, so a token is KPT steps of four instructions and a sum over the row; a block of four
+// waves takes sixteen value channels of a head, D / 16 blocks a head.  A token's r, k, w are read from LDS
+// while the token before it is worked on.
+template <int KPT>
+__global__ __launch_bounds__(256) void wkv_recurrence_rows_kernel(
+    const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
+    const float* __restrict__ z, size_t row, const float* __restrict__ w0, const float* __restrict__ u,
+    float* __restrict__ state, size_t state_row, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ state_slots, float* __restrict__ o, int H, const float* __restrict__ x, int W,
+    size_t prev_off) {
+    constexpr int D = 16 * KPT;
+    constexpr int C = WKV_CHUNK_ELEMS / D;         // tokens a chunk: 16 or 8
+    constexpr int NT = 256;
+    constexpr int EPT = C * D / NT;                // 4
+    constexpr int Q = KPT / 4;
+    __shared__ __attribute__((aligned(16))) float buf[2][3][C * D];       // r, k, w of a chunk, [token][channel]
+    __shared__ float bv[2][C * 16];                                        // v of the block's sixteen channels
+    const int h = blockIdx.x, req = blockIdx.y, tid = threadIdx.x;
+    const int t0 = cu_tokens[req], t1 = cu_tokens[req + 1];
+    if (t1 <= t0) return;
+    const int lane = tid & 63;
+    const int ks = lane & 15, vl = (tid >> 6) * 4 + (lane >> 4), vi = blockIdx.z * 16 + vl;
+    float* srow = state + (size_t)state_slots[req] * state_row;
+    float* S = srow + (size_t)h * D * D;
+    const size_t col = (size_t)h * D;
+    float s[KPT], uu[KPT];
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+        s[i] = S[(size_t)(ks * KPT + i) * D + vi];
+        uu[i] = u[col + ks * KPT + i];
+    }
+    float fr[EPT], fk[EPT], fz[EPT], fv = 0.f;
+    auto fetch = [&](int base) {
+        const int n = min(C, t1 - base);
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+            const int e = tid + i * NT;
+            if (e < n * D) {
+                const size_t a = (size_t)(base + e / D) * row + col + e % D;
+                fr[i] = r[a];
+                fk[i] = k[a];
+                fz[i] = z[a] + w0[col + e % D];
+            }
+        }
+        if (tid < n * 16) fv = v[(size_t)(base + tid / 16) * row + col + blockIdx.z * 16 + tid % 16];
+    };
+    auto stage = [&](int base, int b) {
+        const int n = min(C, t1 - base);
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+            const int e = tid + i * NT;
+            if (e < n * D) {
+                buf[b][0][e] = fr[i];
+                buf[b][1][e] = fk[i];
+                buf[b][2][e] = expf(-expf(fz[i]));
+            }
+        }
+        if (tid < n * 16) bv[b][tid] = fv;
+    };
+    fetch(t0);
+    stage(t0, 0);
+    int b = 0;
+    for (int base = t0; base < t1; base += C, b ^= 1) {
+        const int n = min(C, t1 - base);
+        __syncthreads();
+        if (base + C < t1) fetch(base + C);
+        float4 nr[Q], nk[Q], nw[Q];
+        float nv;
+        auto read = [&](int c) {
+            const float4* cr = reinterpret_cast<const float4*>(buf[b][0] + c * D + ks * KPT);
+            const float4* ck = reinterpret_cast<const float4*>(buf[b][1] + c * D + ks * KPT);
+            const float4* cw = reinterpret_cast<const float4*>(buf[b][2] + c * D + ks * KPT);
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                nr[q] = cr[q];
+                nk[q] = ck[q];
+                nw[q] = cw[q];
+            }
+            nv = bv[b][c * 16 + vl];
+        };
+        read(0);
+        for (int c = 0; c < n; ++c) {
+            float4 cr[Q], ck[Q], cw[Q];
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                cr[q] = nr[q];
+                ck[q] = nk[q];
+                cw[q] = nw[q];
+            }
+            const float vt = nv;
+            if (c + 1 < n) read(c + 1);
+            float acc = 0.f;
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const float rr[4] = {cr[q].x, cr[q].y, cr[q].z, cr[q].w}, kk4[4] = {ck[q].x, ck[q].y, ck[q].z, ck[q].w},
+                            ww[4] = {cw[q].x, cw[q].y, cw[q].z, cw[q].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float kv = kk4[j] * vt;
+                    acc = fmaf(rr[j], fmaf(uu[4 * q + j], kv, s[4 * q + j]), acc);
+                    s[4 * q + j] = fmaf(ww[j], s[4 * q + j], kv);
+                }
+            }
+            acc = row16_sum(acc);
+            if (ks == 0) o[(size_t)(base + c) * H * D + col + vi] = acc;
+        }
+        // (the other buffer was last read before this round's barrier)
+        if (base + C < t1) stage(base + C, b ^ 1);
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) S[(size_t)(ks * KPT + i) * D + vi] = s[i];
+    if (h == 0 && blockIdx.z == 0 && x) {
+        const float* last = x + (size_t)(t1 - 1) * W;
+        for (int c = tid; c < W; c += NT) srow[prev_off + c] = last[c];
+    }
+}
+
 TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, const float* z, size_t row, const float* w0,
                                const float* u, float* state, size_t state_row, const int32_t* cu_tokens,
                                const int32_t* state_slots, float* o, int R, int H, int D, const float* x, int W,
-                               size_t prev_off, tff_stream_t stream) {
+                               size_t prev_off, int long_portions, tff_stream_t stream) {
     TFF_REQUIRE(r && k && v && z && w0 && u && state && cu_tokens && state_slots && o, "wkv_recurrence: null pointer");
     TFF_REQUIRE(R >= 0 && H > 0 && D > 0 && D <= WKV_MAX_D, "wkv_recurrence: %d heads of %d (up to %d)", H, D, WKV_MAX_D);
     TFF_REQUIRE(row >= (size_t)H * D && (size_t)H * D * D <= state_row && (!x || prev_off + (size_t)W <= state_row),
@@ -290,7 +423,15 @@ TFF_API int tff_wkv_recurrence(const float* r, const float* k, const float* v, c
 #define WKV_WAVES(KPT)                                                                                             \
     wkv_recurrence_wave_kernel<KPT><<<grid, 16 * KPT, 0, s>>>(r, k, v, z, row, w0, u, state, state_row, cu_tokens, \
                                                               state_slots, o, H, x, W, prev_off)
-    if (D % 16 == 0) {
+    if (long_portions && (D == 64 || D == 128)) {
+        const dim3 grid3(H, R, D / 16);
+        if (D == 64)
+            wkv_recurrence_rows_kernel<4><<<grid3, 256, 0, s>>>(r, k, v, z, row, w0, u, state, state_row, cu_tokens,
+                                                                state_slots, o, H, x, W, prev_off);
+        else
+            wkv_recurrence_rows_kernel<8><<<grid3, 256, 0, s>>>(r, k, v, z, row, w0, u, state, state_row, cu_tokens,
+                                                                state_slots, o, H, x, W, prev_off);
+    } else if (D % 16 == 0) {
         switch (D / 4) {
             case 4: WKV_WAVES(4); break;
             case 8: WKV_WAVES(8); break;

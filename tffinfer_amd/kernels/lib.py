@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 
 
 class KernelLibraryError(RuntimeError):
@@ -58,7 +58,7 @@ _SIGNATURES = {
     "tff_depth_average": [_P, _Z, _I, _P, _P, _P, _Z, _I, _P],
     "tff_scale_rows": [_P, _F, _Z, _P],
     "tff_token_shift_mix": [_P, _P, _Z, _Z, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P],
-    "tff_wkv_recurrence": [_P, _P, _P, _P, _Z, _P, _P, _P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _Z, _P],
+    "tff_wkv_recurrence": [_P, _P, _P, _P, _Z, _P, _P, _P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _Z, _I, _P],
     "tff_head_norm_gate": [_P, _P, _Z, _P, _F, _P, _I, _I, _I, _I, _P],
     "tff_tanh": [_P, _P, _Z, _I, _P],
     "tff_qk_bias_norm_store": [_P, _Z, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],

@@ -1198,6 +1198,10 @@ def token_shift_mix(x: torch.Tensor, state: torch.Tensor, prev_off: int, mu: tor
     return out
 
 
+#: tokens of a step's longest entry from which the recurrence runs in its form for prompts
+WKV_LONG_PORTION = 16
+
+
 def wkv_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, w0: torch.Tensor,
                    u: torch.Tensor, state: torch.Tensor, batch, H: int, D: int, x: torch.Tensor | None = None,
                    prev_off: int = 0) -> torch.Tensor:
@@ -1231,7 +1235,8 @@ def wkv_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.T
     _lib.check(_lib.load().tff_wkv_recurrence(r.data_ptr(), k.data_ptr(), v.data_ptr(), z.data_ptr(), r.stride(0),
                                               w0.data_ptr(), u.data_ptr(), state.data_ptr(), row,
                                               batch.cu_tokens.data_ptr(), batch.state_slots.data_ptr(), o.data_ptr(),
-                                              batch.num_reqs, H, D, _ptr(x), W, int(prev_off), _stream()))
+                                              batch.num_reqs, H, D, _ptr(x), W, int(prev_off),
+                                              1 if getattr(batch, "max_new_tokens", 0) >= WKV_LONG_PORTION else 0, _stream()))
     return o
 
 
