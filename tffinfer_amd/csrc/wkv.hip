@@ -264,7 +264,7 @@ __global__ __launch_bounds__(512) void wkv_recurrence_wave_kernel(
             acc = rows_sum(acc);        // (quarter 0 + quarter 1) + (quarter 2 + quarter 3), in every lane
             if (ks == 0) o[(size_t)(base + c) * H * D + col + vi] = acc;
         }
-        // (the other buffer was last read before this round's barrier)
+        // (the other buffer was last read before this pass's barrier)
         if (base + C < t1) stage(base + C, b ^ 1);
     }
 #pragma unroll
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256) void wkv_recurrence_rows_kernel(
             acc = row16_sum(acc);
             if (ks == 0) o[(size_t)(base + c) * H * D + col + vi] = acc;
         }
-        // (the other buffer was last read before this round's barrier)
+        // (the other buffer was last read before this pass's barrier)
         if (base + C < t1) stage(base + C, b ^ 1);
     }
 #pragma unroll
