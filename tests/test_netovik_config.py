@@ -98,12 +98,12 @@ def test_round_trip_and_refusals(tmp_path):
     for breaker, text in (
             (lambda c: c["layers"][0].update(type="other"), "mixer"),
             (lambda c: c["layers"][1]["mlp"].update(kind="sparse"), "feed-forward"),
-            (lambda c: c["layers"][0]["mixer"].pop("softcap"), "softcap"),
+            (lambda c: c["layers"][0]["mixer"].pop("scale"), "scale"),
             (lambda c: c["layers"][0]["mixer"].update(vdim=24), "values are the keys"),
             (lambda c: c["layers"][0]["mixer"].update(kv_heads=3), "kv heads"),
             (lambda c: c["layers"][1]["mixer"].update(dim=300), "128"),
             (lambda c: c["norm"].update(groups=5), "groups"),
-            (lambda c: c.pop("embedding"), "embedding"),
+            (lambda c: c.update(embedding=3), "embedding"),
             (lambda c: c["layers"][1]["mlp"]["router"].update(top=9), "top")):
         bad = copy.deepcopy(NV_A)
         breaker(bad)

@@ -520,3 +520,41 @@ def test_a_preempted_request_starts_its_state_again(netovik_dirs):
         preempted.append(sum(r.num_preemptions for r in res))
     assert outs[0] == outs[1]
     assert preempted[0] == 0 and preempted[1] > 0
+
+
+def test_the_command_line_with_a_configuration_file_of_this_architecture(tmp_path):
+    """--config FILE --random-weights through bin/tffinfer: the weights are those of the folder that
+    --save-model writes, the dumped rows are the logits that chose each token; a pool so small that
+    requests are preempted and computed again gives the same tokens."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from netovik_models import NV_C
+    prog = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "tffinfer")
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(NV_C))
+    folder, dump = str(tmp_path / "nvC"), str(tmp_path / "logits.f32")
+    common = [sys.executable, prog, "--config", str(cfg), "--random-weights", "--seed", "5", "--fp32", "--n-ctx", "256",
+              "--n-predict", "12", "--ignore-eos", "--json", "--random-prompts", "3:30", "--page-size", "8",
+              "--max-batches", "3"]
+    p = subprocess.run(common + ["--save-model", folder, "--dump-logits", dump, "--kv-tokens", "512"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    recs = [json.loads(ln) for ln in p.stdout.strip().splitlines()]
+    meta = json.load(open(dump + ".json"))
+    V = NV_C["vocab"]
+    rows = np.fromfile(dump, dtype="<f4").reshape(meta["shape"])
+    assert meta["shape"] == [36, V]
+    for i, r in enumerate(recs):
+        ref = oracle_logits(folder, r["prompt"] + r["output"])
+        first = meta["requests"][i]["first_row"]
+        for j, tok in enumerate(r["output"]):
+            row = torch.from_numpy(rows[first + j].copy())
+            assert rel_err(row, ref[len(r["prompt"]) - 1 + j]) <= tol("float32", "nvC")
+            assert tok == int(torch.argmax(row))
+    tight = subprocess.run(common + ["--num-pages", "11"], capture_output=True, text=True, timeout=300)
+    assert tight.returncode == 0, tight.stderr[-3000:]
+    assert "preemption" in tight.stderr
+    assert [json.loads(ln)["output"] for ln in tight.stdout.strip().splitlines()] == [r["output"] for r in recs]

@@ -51,7 +51,7 @@ def _mixer_spec(i: int, width: int, eps: float, kind: str, m) -> PartSpec:
             "head_dim": require(m, "dim", int, where),
             "value_dim": optional(m, "vdim", int, None, where),
             "scale": require(m, "scale", float, where),
-            "softcap": require(m, "softcap", float, where),
+            "softcap": optional(m, "softcap", float, None, where),      # (none: the scores as they are)
             "bias_max": require(m, "bias_max", int, where),
             "bias_buckets": optional(m, "bias_buckets", int, None, where),
             "window": window,
@@ -112,8 +112,10 @@ class NetovikConfig(ModelConfig):
         norm, emb = d.get("norm"), d.get("embedding")
         if not isinstance(norm, dict):
             raise ConfigError("config.json: required object 'norm' is missing")
+        if emb is None:
+            emb = {}            # (no scale: the rows as they are)
         if not isinstance(emb, dict):
-            raise ConfigError("config.json: required object 'embedding' is missing")
+            raise ConfigError("config.json: 'embedding' must be an object")
         eos = d.get("eos_token_id")
         known = {"architecture", "architectures", "layers", "norm", "embedding", "vocab", "width",
                  "max_position_embeddings", "eos_token_id"}
