@@ -377,6 +377,245 @@ __global__ __launch_bounds__(64) void mixed_attention_merge_kernel(const float* 
     }
 }
 
+// ---- prompts in bfloat16: sixteen queries a block, the two products on the matrix cores ----
+//
+// A block takes up to 16 consecutive tokens of one request (a work item: first token, count) and all heads.
+// Per tile of 16 keys (borders at multiples of 16 from the sequence's start):
+//   1. S_g = Q_g K^T per head g: MFMA 16x16x32 over the head's elements, a wave a head at a time, operands straight
+//      from memory (lane (row, quarter) holds 8 consecutive elements of its row); scale, cap and bias on the
+//      accumulators; the scores go to LDS as float32 [head][query][key].
+//   2. A thread per (head, query): the scores of all heads mixed, the mask, the running maximum and sum, the
+//      weights to LDS as bfloat16 [head][query][key].
+//   3. O_h += P_h V: MFMA 16x16x32 whose upper sixteen contraction slots are zero; values from the transposed
+//      pages (a tile lies in one page: pages of a multiple of 16 tokens).
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 ma_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ma_floatx4;
+
+#define Q16_THREADS 512
+#define Q16_WAVES 8
+#define Q16_SROW 16      // floats a (head, query) row of scores takes in LDS
+// Where key chunk c (four keys) of query qq lies in its row: rows lie 64 bytes apart, so without this the rows of
+// every other query would meet in the same banks when sixteen threads read their own query's chunk c.
+#define Q16_CHUNK(c, qq) (((c) ^ (((qq) >> 1) & 3)) * 4)
+
+template <int HPW, int EB>
+__global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int bt_width, const int32_t* __restrict__ token_req,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ work, const float* __restrict__ bias,
+    int bias_rows, const float* __restrict__ mix, float scale, float cap, int window, int keep_first, int sink,
+    bf16_t* __restrict__ out, int H, int G, int page_size) {
+    constexpr int D = EB * 16, KC = D / 32;
+    extern __shared__ float lds[];
+    float* s_raw = lds;                                  // [H][16][Q16_SROW]
+    float* mix_s = s_raw + H * 16 * Q16_SROW;            // [H][H] (if mix)
+    float* m_s = mix_s + (mix ? (H * H + 3) / 4 * 4 : 0);  // [H][16] (16-byte aligned, as all that follows)
+    float* l_s = m_s + H * 16;
+    float* c_s = l_s + H * 16;
+    bf16_t* p_s = reinterpret_cast<bf16_t*>(c_s + H * 16);   // [H][16][16]
+    const int t0 = work[2 * blockIdx.x], n = work[2 * blockIdx.x + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, col = lane & 15, g4 = lane >> 4;
+    const int pos0 = positions[t0], pos_last = pos0 + n - 1;
+    const int32_t* table = block_tables + (size_t)token_req[t0] * bt_width;
+    const int rep = H / G, HD = H * D;
+    if (mix)
+        for (int i = tid; i < H * H; i += Q16_THREADS) mix_s[i] = mix[i];
+    for (int i = tid; i < H * 16; i += Q16_THREADS) {
+        m_s[i] = sink ? 0.f : -INFINITY;
+        l_s[i] = sink ? 1.f : 0.f;
+    }
+    ma_floatx4 oacc[HPW][EB];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+        for (int eb = 0; eb < EB; ++eb) oacc[hh][eb] = ma_floatx4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* qrow = q + (size_t)(t0 + min(col, n - 1)) * HD + g4 * 8;
+    const size_t page_elems = (size_t)G * D * page_size;
+    __syncthreads();
+
+    auto tile = [&](int jt) {
+        // 1. scores
+        {
+            const int j = min(jt + col, pos_last);
+            const bf16_t* kpage = k_cache + (size_t)table[j / page_size] * page_elems + (size_t)(j % page_size) * D + g4 * 8;
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = wv + hh * Q16_WAVES;
+                if (h < H) {
+                    const bf16_t* krow = kpage + (size_t)(h / rep) * page_size * D;
+                    ma_floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kc = 0; kc < KC; ++kc) {
+                        const ma_bf16x8 a = *reinterpret_cast<const ma_bf16x8*>(qrow + h * D + kc * 32);
+                        const ma_bf16x8 b = *reinterpret_cast<const ma_bf16x8*>(krow + kc * 32);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {        // (query g4 * 4 + i, key col)
+                        const int qq = g4 * 4 + i;
+                        float sc = acc[i] * scale;
+                        if (cap > 0.f) sc = cap * tanhf(sc / cap);
+                        if (bias) sc += bias[(size_t)min(max(pos0 + qq - (jt + col), 0), bias_rows - 1) * H + h];
+                        s_raw[(h * 16 + qq) * Q16_SROW + Q16_CHUNK(col >> 2, qq) + (col & 3)] = sc;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // 2. a thread per (head, query)
+        {
+            const int h = tid >> 4, qq = tid & 15;
+            if (h < H) {
+                float sm[16];
+                if (mix) {
+#pragma unroll
+                    for (int kk = 0; kk < 16; ++kk) sm[kk] = 0.f;
+                    for (int g = 0; g < H; ++g) {
+                        const float tg = mix_s[h * H + g];
+                        const float4* row = reinterpret_cast<const float4*>(s_raw + (g * 16 + qq) * Q16_SROW);
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            const float4 v4 = row[Q16_CHUNK(c, qq) >> 2];
+                            sm[4 * c] = fmaf(tg, v4.x, sm[4 * c]);
+                            sm[4 * c + 1] = fmaf(tg, v4.y, sm[4 * c + 1]);
+                            sm[4 * c + 2] = fmaf(tg, v4.z, sm[4 * c + 2]);
+                            sm[4 * c + 3] = fmaf(tg, v4.w, sm[4 * c + 3]);
+                        }
+                    }
+                } else {
+                    const float4* row = reinterpret_cast<const float4*>(s_raw + (h * 16 + qq) * Q16_SROW);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float4 v4 = row[Q16_CHUNK(c, qq) >> 2];
+                        sm[4 * c] = v4.x; sm[4 * c + 1] = v4.y; sm[4 * c + 2] = v4.z; sm[4 * c + 3] = v4.w;
+                    }
+                }
+                const int posq = pos0 + qq;
+                const float m_old = m_s[h * 16 + qq];
+                float mx = m_old;
+                bool vis[16];
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) {
+                    const int j = jt + kk;
+                    vis[kk] = qq < n && j <= posq && (window <= 0 || posq - j < window || j < keep_first);
+                    if (vis[kk]) mx = fmaxf(mx, sm[kk]);
+                }
+                float corr = 1.f, sum = 0.f;
+                if (mx > -INFINITY) corr = expf(m_old - mx);
+                union { bf16_t h[16]; uint4 u[2]; } pk;
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) {
+                    // (the sum takes the weights as the product will see them)
+                    const bf16_t pb = (bf16_t)(vis[kk] ? expf(sm[kk] - mx) : 0.f);
+                    pk.h[kk] = pb;
+                    sum += (float)pb;
+                }
+                m_s[h * 16 + qq] = mx;
+                l_s[h * 16 + qq] = l_s[h * 16 + qq] * corr + sum;
+                c_s[h * 16 + qq] = corr;
+                uint4* pd = reinterpret_cast<uint4*>(p_s + (h * 16 + qq) * 16);
+                pd[0] = pk.u[0];
+                pd[1] = pk.u[1];
+            }
+        }
+        __syncthreads();
+        // 3. weighted values
+        {
+            const bf16_t* vpage = v_cache + (size_t)table[jt / page_size] * page_elems + (size_t)col * page_size + jt % page_size + g4 * 8;
+            const ma_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = wv + hh * Q16_WAVES;
+                if (h < H) {
+                    const ma_bf16x8 a = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(p_s + (h * 16 + col) * 16 + g4 * 8) : zero;
+                    float cr[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) cr[i] = c_s[h * 16 + g4 * 4 + i];
+                    const bf16_t* vhead = vpage + (size_t)(h / rep) * D * page_size;
+#pragma unroll
+                    for (int eb = 0; eb < EB; ++eb) {
+                        const ma_bf16x8 b = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(vhead + (size_t)eb * 16 * page_size) : zero;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) oacc[hh][eb][i] *= cr[i];
+                        oacc[hh][eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, oacc[hh][eb], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // (the next tile's scores go to s_raw, which nobody reads any more; its first barrier stands between these
+        // reads of p_s and c_s and their next writes)
+    };
+
+    const int lo_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int lo_last = window > 0 ? max(0, pos_last - window + 1) : 0;
+    const int jt_b = (lo_first / 16) * 16;
+    for (int jt = 0; jt < min(min(keep_first, lo_last), jt_b); jt += 16) tile(jt);      // kept first tokens before the windows
+    for (int jt = jt_b; jt <= pos_last; jt += 16) tile(jt);
+    __syncthreads();
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        const int h = wv + hh * Q16_WAVES;
+        if (h < H) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int qq = g4 * 4 + i;
+                if (qq < n) {
+                    const float l = l_s[h * 16 + qq];
+                    const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+                    for (int eb = 0; eb < EB; ++eb)
+                        out[(size_t)(t0 + qq) * HD + h * D + eb * 16 + col] = (bf16_t)(oacc[hh][eb][i] * inv);
+                }
+            }
+        }
+    }
+}
+
+static size_t q16_lds_bytes(int H, bool mix) {
+    return sizeof(float) * ((size_t)H * 16 * Q16_SROW + (mix ? ((size_t)H * H + 3) / 4 * 4 : 0) + 3 * (size_t)H * 16) + 2 * (size_t)H * 256;
+}
+
+// bfloat16, up to 32 heads of 32, 64 or 128 elements, pages of a multiple of 16 tokens.
+TFF_API int tff_mixed_attention_q16_supported(int H, int D, int page_size, int has_mix) {
+    return H > 0 && H <= 32 && (D == 32 || D == 64 || D == 128) && page_size % 16 == 0 &&
+           q16_lds_bytes(H, has_mix != 0) <= 64 * 1024;
+}
+
+// work: int32 [items][2] = (first token of the step, count <= 16), the tokens of an item consecutive tokens of one
+// request.
+TFF_API int tff_mixed_attention_q16(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                    int bt_width, const int32_t* token_req, const int32_t* positions, const int32_t* work,
+                                    int items, const float* bias, int bias_rows, const float* mix, float scale, float cap,
+                                    int window, int keep_first, int sink, void* out, int H, int G, int D, int page_size,
+                                    tff_stream_t stream) {
+    TFF_REQUIRE(q && k_cache && v_cache && block_tables && token_req && positions && work && out,
+                "mixed_attention_q16: null pointer");
+    TFF_REQUIRE(G > 0 && H % G == 0 && bt_width > 0 && tff_mixed_attention_q16_supported(H, D, page_size, mix != nullptr),
+                "mixed_attention_q16: %d heads of %d on %d kv heads, pages of %d", H, D, G, page_size);
+    TFF_REQUIRE(!bias || bias_rows > 0, "mixed_attention_q16: a bias table without rows");
+    TFF_REQUIRE(window >= 0 && keep_first >= 0 && items >= 0, "mixed_attention_q16: negative sizes");
+    if (items == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t lds = q16_lds_bytes(H, mix != nullptr);
+    const int hpw = (H + Q16_WAVES - 1) / Q16_WAVES;
+#define Q16_LAUNCH(HPW, EB)                                                                                          \
+    mixed_attention_q16_kernel<HPW, EB><<<items, Q16_THREADS, lds, s>>>(                                            \
+        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_width, token_req,       \
+        positions, work, bias, bias_rows, mix, scale, cap, window, keep_first, sink, (bf16_t*)out, H, G, page_size)
+#define Q16_BY_EB(HPW)                  \
+    do {                                \
+        if (D == 32) Q16_LAUNCH(HPW, 2); \
+        else if (D == 64) Q16_LAUNCH(HPW, 4); \
+        else Q16_LAUNCH(HPW, 8);        \
+    } while (0)
+    if (hpw <= 1) Q16_BY_EB(1);
+    else if (hpw <= 2) Q16_BY_EB(2);
+    else Q16_BY_EB(4);
+#undef Q16_BY_EB
+#undef Q16_LAUNCH
+    return tff_check_launch("mixed_attention_q16");
+}
+
 static size_t ma_lds_bytes(int H, int D, bool mix) {
     return sizeof(float) * ((size_t)H * D + 2 * (size_t)H * MA_TK + (mix ? (size_t)H * H : 0) + 3 * (size_t)H + MA_TK / 2);
 }

@@ -1291,6 +1291,8 @@ def qk_bias_norm_store(qk: torch.Tensor, q_bias, k_bias, eps: float, H: int, G: 
 
 #: blocks a step of few tokens spreads its attention over (two a CU)
 MIXED_ATTENTION_BLOCKS = 512
+#: tokens of a step from which bfloat16 attention runs sixteen queries a block on the matrix cores
+MIXED_ATTENTION_Q16_TOKENS = 64
 
 
 def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: float, softcap: float = 0.0,
@@ -1327,6 +1329,21 @@ def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: f
     if batch.token_req.numel() < T or batch.positions.numel() < T:
         raise _lib.KernelError("mixed_attention: the step's tables are shorter than q")
     out = torch.empty(T, H * D, dtype=dt, device=q.device)
+    cu = getattr(batch, "host_cu_tokens", None)
+    if (splits is None and dt == torch.bfloat16 and cu is not None and T >= MIXED_ATTENTION_Q16_TOKENS
+            and getattr(batch, "max_new_tokens", 0) >= 16
+            and L.tff_mixed_attention_q16_supported(H, D, kv.page_size, 1 if mix is not None else 0)):
+        # a prompt's portions: sixteen queries a block, the products on the matrix cores
+        cache = getattr(batch, "_q16_work", None)
+        if cache is None:
+            items = [(t, min(16, cu[r + 1] - t)) for r in range(len(cu) - 1) for t in range(cu[r], cu[r + 1], 16)]
+            cache = batch._q16_work = _staging.send(q.device, [np.asarray(items, dtype=np.int32).reshape(-1, 2)])[0]
+        _lib.check(L.tff_mixed_attention_q16(q.data_ptr(), kv.k_cache.data_ptr(), kv.v_cache.data_ptr(), bt.data_ptr(),
+                                             bt.shape[1], batch.token_req.data_ptr(), batch.positions.data_ptr(),
+                                             cache.data_ptr(), cache.shape[0], _ptr(bias), rows, _ptr(mix), float(scale),
+                                             float(softcap), int(window), int(keep_first), 1 if sink else 0,
+                                             out.data_ptr(), H, G, D, kv.page_size, _stream()))
+        return out
     # tiles of 64 keys that a token of this step can have at most (what the block tables can hold, or the window
     # and the kept tokens): a size the host knows without reading a position, so a captured step keeps it
     reach = bt.shape[1] * kv.page_size
