@@ -434,22 +434,41 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     __syncthreads();
 
     auto tile = [&](int jt) {
-        // 1. scores
+        // 1. scores: the wave's heads lie side by side, so they mostly share a kv head and its keys are fetched once;
+        // all of a tile's operands are asked for before the first product
         {
             const int j = min(jt + col, pos_last);
             const bf16_t* kpage = k_cache + (size_t)table[j / page_size] * page_elems + (size_t)(j % page_size) * D + g4 * 8;
+            // (the queries of all the wave's heads at once where the registers hold them beside the results)
+            constexpr bool Q_AHEAD = HPW * KC <= 8;
+            ma_bf16x8 qf[Q_AHEAD ? HPW : 1][KC], kf[KC];
+            if (Q_AHEAD) {
+#pragma unroll
+                for (int hh = 0; hh < HPW; ++hh) {
+                    const int h = min(wv * HPW + hh, H - 1);
+#pragma unroll
+                    for (int kc = 0; kc < KC; ++kc) qf[Q_AHEAD ? hh : 0][kc] = *reinterpret_cast<const ma_bf16x8*>(qrow + h * D + kc * 32);
+                }
+            }
+            int kv_have = -1;
 #pragma unroll
             for (int hh = 0; hh < HPW; ++hh) {
-                const int h = wv + hh * Q16_WAVES;
+                const int h = wv * HPW + hh;
                 if (h < H) {
-                    const bf16_t* krow = kpage + (size_t)(h / rep) * page_size * D;
+                    if (h / rep != kv_have) {
+                        kv_have = h / rep;
+                        const bf16_t* krow = kpage + (size_t)kv_have * page_size * D;
+#pragma unroll
+                        for (int kc = 0; kc < KC; ++kc) kf[kc] = *reinterpret_cast<const ma_bf16x8*>(krow + kc * 32);
+                    }
+                    if (!Q_AHEAD) {
+#pragma unroll
+                        for (int kc = 0; kc < KC; ++kc) qf[0][kc] = *reinterpret_cast<const ma_bf16x8*>(qrow + h * D + kc * 32);
+                    }
                     ma_floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int kc = 0; kc < KC; ++kc) {
-                        const ma_bf16x8 a = *reinterpret_cast<const ma_bf16x8*>(qrow + h * D + kc * 32);
-                        const ma_bf16x8 b = *reinterpret_cast<const ma_bf16x8*>(krow + kc * 32);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-                    }
+                    for (int kc = 0; kc < KC; ++kc)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[Q_AHEAD ? hh : 0][kc], kf[kc], acc, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {        // (query g4 * 4 + i, key col)
                         const int qq = g4 * 4 + i;
@@ -519,25 +538,40 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
             }
         }
         __syncthreads();
-        // 3. weighted values
+        // 3. weighted values; where the wave's heads share a kv head its values are fetched once for all of them
         {
             const bf16_t* vpage = v_cache + (size_t)table[jt / page_size] * page_elems + (size_t)col * page_size + jt % page_size + g4 * 8;
             const ma_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+            const int h_lo = wv * HPW, h_hi = min(h_lo + HPW, H) - 1;
+            const bool one_kv = h_lo < H && h_lo / rep == h_hi / rep;
+            constexpr int VG = HPW * EB >= 32 ? 2 : (EB < 4 ? EB : 4);      // value fragments asked for at a time (fewer where the results fill the registers)
 #pragma unroll
-            for (int hh = 0; hh < HPW; ++hh) {
-                const int h = wv + hh * Q16_WAVES;
-                if (h < H) {
-                    const ma_bf16x8 a = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(p_s + (h * 16 + col) * 16 + g4 * 8) : zero;
-                    float cr[4];
+            for (int e0 = 0; e0 < EB; e0 += VG) {
+                ma_bf16x8 vb[VG];
+                if (one_kv) {
+                    const bf16_t* vhead = vpage + (size_t)(h_lo / rep) * D * page_size;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) cr[i] = c_s[h * 16 + g4 * 4 + i];
-                    const bf16_t* vhead = vpage + (size_t)(h / rep) * D * page_size;
+                    for (int e = 0; e < VG; ++e)
+                        vb[e] = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(vhead + (size_t)(e0 + e) * 16 * page_size) : zero;
+                }
 #pragma unroll
-                    for (int eb = 0; eb < EB; ++eb) {
-                        const ma_bf16x8 b = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(vhead + (size_t)eb * 16 * page_size) : zero;
+                for (int hh = 0; hh < HPW; ++hh) {
+                    const int h = h_lo + hh;
+                    if (h < H) {
+                        const bf16_t* vhead = vpage + (size_t)(h / rep) * D * page_size;
+                        // (the head's weights and factors come from LDS again for every group: registers are dearer)
+                        const ma_bf16x8 pa = g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(p_s + (h * 16 + col) * 16 + g4 * 8) : zero;
+                        float cr[4];
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) oacc[hh][eb][i] *= cr[i];
-                        oacc[hh][eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, oacc[hh][eb], 0, 0, 0);
+                        for (int i = 0; i < 4; ++i) cr[i] = c_s[h * 16 + g4 * 4 + i];
+#pragma unroll
+                        for (int e = 0; e < VG; ++e) {
+                            const ma_bf16x8 b = one_kv ? vb[e]
+                                                       : (g4 < 2 ? *reinterpret_cast<const ma_bf16x8*>(vhead + (size_t)(e0 + e) * 16 * page_size) : zero);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) oacc[hh][e0 + e][i] *= cr[i];
+                            oacc[hh][e0 + e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, b, oacc[hh][e0 + e], 0, 0, 0);
+                        }
                     }
                 }
             }
@@ -554,7 +588,7 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     __syncthreads();
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
-        const int h = wv + hh * Q16_WAVES;
+        const int h = wv * HPW + hh;
         if (h < H) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
