@@ -61,10 +61,11 @@ NV_B = model(96, 257, 1, 1e-5, 1.0, [
     layer(att(1, 1, 40, 0.2, 5.0, 100, 32, window=8, keep=9), dense(40)),
     layer(wkv(12, 8, rank=16), dense(104)),
 ])
-# two attention layers in a row with different caches, one without a window; both experts chosen; three groups
+# two attention layers in a row with different caches, one without a window and with heads of 32 (in bfloat16 its
+# prompts run on the matrix cores); both experts chosen; three groups
 NV_C = model(72, 128, 3, 1e-4, 1.9, [
     layer(att(12, 4, 8, 0.4, 50.0, 64, 16, window=70, keep=2), moe(2, 2, 16)),
-    layer(att(6, 1, 16, 0.25, 12.0, 33, 8), dense(40)),
+    layer(att(6, 2, 32, 0.18, 12.0, 33, 8), dense(40)),
     layer(wkv(3, 24), dense(48)),
 ])
 # recurrence only; one expert a token

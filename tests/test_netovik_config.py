@@ -42,7 +42,7 @@ def test_every_size_and_constant_comes_from_the_file():
     assert isinstance(n, GroupRMSNorm) and (n.groups, n.eps, n.size) == (2, 1e-6, 64)
     # a layer without a window keeps every key; kv heads default to the heads
     c = build_model_skeleton(config_from_dict(copy.deepcopy(NV_C)))
-    assert c.blocks[1].mixer.cache_spec() == KVCacheSpec(1, 16, 0, 0)
+    assert c.blocks[1].mixer.cache_spec() == KVCacheSpec(2, 32, 0, 0)
     m = copy.deepcopy(NV_C)
     del m["layers"][0]["mixer"]["kv_heads"]
     assert build_model_skeleton(config_from_dict(m)).blocks[0].mixer.num_kv_heads == 12

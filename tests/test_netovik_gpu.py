@@ -561,3 +561,19 @@ def test_the_command_line_with_a_configuration_file_of_this_architecture(tmp_pat
     assert tight.returncode == 0, tight.stderr[-3000:]
     assert "preemption" in tight.stderr
     assert [json.loads(ln)["output"] for ln in tight.stdout.strip().splitlines()] == [r["output"] for r in recs]
+
+
+@pytest.mark.parametrize("mode", ["chunks", "mixed"])
+def test_prompt_attention_on_the_matrix_cores_beside_single_tokens(netovik_dirs, mode, monkeypatch):
+    """Steps in which a prompt's portion of 16 tokens and more stands beside other requests' single tokens and
+    short portions, all run by the kernel for prompts (its threshold on a step's tokens lowered for the test)."""
+    ops = _ops()
+    monkeypatch.setattr(ops, "MIXED_ATTENTION_Q16_TOKENS", 16)
+    model_dir = netovik_dirs["nvC"]
+    reqs = requests_for("nvC", model_dir)
+    steps = {"chunks": rl.trace_chunks, "mixed": rl.trace_mixed}[mode](reqs)
+    assert any(max(len(e["tokens"]) for e in s["entries"]) >= 16 and len(s["entries"]) > (1 if mode == "mixed" else 0) for s in steps)
+    ps = NETOVIK_PAGE["nvC"]
+    runner = make_runner(model_dir, "bfloat16", ps, rl.max_live_tokens(steps, unit=ps) // ps)
+    results = rl.run_steps_in_process(runner, steps)
+    check(model_dir, reqs, steps, results, "bfloat16", "nvC")
