@@ -219,7 +219,7 @@ def _plain_attention(qk, qb, kb, H, G, D, eps, **kw):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,page", [(4, 2, 16, 16), (3, 3, 8, 8), (12, 4, 8, 32), (1, 1, 40, 8), (6, 1, 64, 16), (5, 5, 12, 16),
-                                        (5, 5, 32, 16), (32, 8, 128, 32), (9, 3, 64, 8)])
+                                        (5, 5, 32, 16), (32, 8, 128, 32), (9, 3, 64, 8), (16, 16, 32, 16), (12, 4, 64, 16), (20, 2, 32, 32)])
 def test_attention_with_every_term(H, G, D, page, dtype):
     """Bias, cap, exchange between heads, window with kept first tokens and the 1 in the denominator, on a
     prompt in one step and on the same tokens as a prompt's portion followed by single tokens; then each
