@@ -175,7 +175,7 @@ __global__ __launch_bounds__(MA_THREADS) void mixed_attention_kernel(
     __syncthreads();
     const MaTiles tiles(pos, window, keep_first);
     const int i_lo = nsplit == 1 ? 0 : split * tiles_per_split;
-    const int i_hi = nsplit == 1 ? tiles.n : min(tiles.n, i_lo + tiles_per_split);
+    const int i_hi = split == nsplit - 1 ? tiles.n : min(tiles.n, i_lo + tiles_per_split);      // (the last split takes what is left)
     // lanes of a key: a key's row of D elements is read by D / 8 neighbouring lanes, 16 bytes each (where D / 8
     // is a power of two up to 64), so that a wave's load covers whole rows; else a lane reads a key's whole row
     const int lpk = D / 8;
@@ -404,7 +404,8 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     const int32_t* __restrict__ block_tables, int bt_width, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ work, const float* __restrict__ bias,
     int bias_rows, const float* __restrict__ mix, float scale, float cap, int window, int keep_first, int sink,
-    bf16_t* __restrict__ out, int H, int G, int page_size) {
+    bf16_t* __restrict__ out, int H, int G, int page_size, int tiles_per_split, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
     constexpr int D = EB * 16, KC = D / 32;
     extern __shared__ float lds[];
     float* s_raw = lds;                                  // [H][16][Q16_SROW]
@@ -414,6 +415,8 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     float* c_s = l_s + H * 16;
     bf16_t* p_s = reinterpret_cast<bf16_t*>(c_s + H * 16);   // [H][16][16]
     const int t0 = work[2 * blockIdx.x], n = work[2 * blockIdx.x + 1];
+    const int split = blockIdx.y, nsplit = gridDim.y;
+    const bool own_sink = sink && nsplit == 1;       // (with several splits the merge adds the sink's term)
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, col = lane & 15, g4 = lane >> 4;
     const int pos0 = positions[t0], pos_last = pos0 + n - 1;
     const int32_t* table = block_tables + (size_t)token_req[t0] * bt_width;
@@ -421,8 +424,8 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     if (mix)
         for (int i = tid; i < H * H; i += Q16_THREADS) mix_s[i] = mix[i];
     for (int i = tid; i < H * 16; i += Q16_THREADS) {
-        m_s[i] = sink ? 0.f : -INFINITY;
-        l_s[i] = sink ? 1.f : 0.f;
+        m_s[i] = own_sink ? 0.f : -INFINITY;
+        l_s[i] = own_sink ? 1.f : 0.f;
     }
     ma_floatx4 oacc[HPW][EB];
 #pragma unroll
@@ -583,8 +586,12 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
     const int lo_first = window > 0 ? max(0, pos0 - window + 1) : 0;
     const int lo_last = window > 0 ? max(0, pos_last - window + 1) : 0;
     const int jt_b = (lo_first / 16) * 16;
-    for (int jt = 0; jt < min(min(keep_first, lo_last), jt_b); jt += 16) tile(jt);      // kept first tokens before the windows
-    for (int jt = jt_b; jt <= pos_last; jt += 16) tile(jt);
+    // the block's tiles, numbered through: those of the kept first tokens before the windows, then the windows'
+    const int n_a = (min(min(keep_first, lo_last), jt_b) + 15) / 16;
+    const int tiles = n_a + (pos_last - jt_b) / 16 + 1;
+    const int i_lo = nsplit == 1 ? 0 : split * tiles_per_split;
+    const int i_hi = split == nsplit - 1 ? tiles : min(tiles, i_lo + tiles_per_split);      // (the last split takes what is left)
+    for (int ti = i_lo; ti < i_hi; ++ti) tile(ti < n_a ? ti * 16 : jt_b + (ti - n_a) * 16);
     __syncthreads();
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
@@ -594,13 +601,28 @@ __global__ __launch_bounds__(Q16_THREADS) void mixed_attention_q16_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int qq = g4 * 4 + i;
                 if (qq < n) {
-                    const float l = l_s[h * 16 + qq];
-                    const float inv = l > 0.f ? 1.0f / l : 0.f;
+                    if (nsplit == 1) {
+                        const float l = l_s[h * 16 + qq];
+                        const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
-                    for (int eb = 0; eb < EB; ++eb)
-                        out[(size_t)(t0 + qq) * HD + h * D + eb * 16 + col] = (bf16_t)(oacc[hh][eb][i] * inv);
+                        for (int eb = 0; eb < EB; ++eb)
+                            out[(size_t)(t0 + qq) * HD + h * D + eb * 16 + col] = (bf16_t)(oacc[hh][eb][i] * inv);
+                    } else {
+                        float* po = part_o + ((size_t)(t0 + qq) * nsplit + split) * HD + h * D + col;
+#pragma unroll
+                        for (int eb = 0; eb < EB; ++eb) po[eb * 16] = oacc[hh][eb][i];
+                    }
                 }
             }
+        }
+    }
+    if (nsplit > 1) {
+        // (maximum and sum per head and query, in the merge's layout: [token][split][maxima of the heads | sums])
+        const int h = tid >> 4, qq = tid & 15;
+        if (h < H && qq < n) {
+            float* pm = part_ml + ((size_t)(t0 + qq) * nsplit + split) * 2 * H;
+            pm[h] = m_s[h * 16 + qq];
+            pm[H + h] = l_s[h * 16 + qq];
         }
     }
 }
@@ -616,14 +638,17 @@ TFF_API int tff_mixed_attention_q16_supported(int H, int D, int page_size, int h
 }
 
 // work: int32 [items][2] = (first token of the step, count <= 16), the tokens of an item consecutive tokens of one
-// request.
+// request; every one of the step's T tokens lies in one item.  splits > 1: an item's tiles of 16 keys are dealt to
+// `splits` blocks, tiles_per_split each, and merged as tff_mixed_attention's are (the same workspace size).
 TFF_API int tff_mixed_attention_q16(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                     int bt_width, const int32_t* token_req, const int32_t* positions, const int32_t* work,
                                     int items, const float* bias, int bias_rows, const float* mix, float scale, float cap,
-                                    int window, int keep_first, int sink, void* out, int H, int G, int D, int page_size,
-                                    tff_stream_t stream) {
+                                    int window, int keep_first, int sink, void* out, int T, int H, int G, int D,
+                                    int page_size, int splits, int tiles_per_split, float* workspace, tff_stream_t stream) {
     TFF_REQUIRE(q && k_cache && v_cache && block_tables && token_req && positions && work && out,
                 "mixed_attention_q16: null pointer");
+    TFF_REQUIRE(splits >= 1 && splits <= 65535 && (splits == 1 || (tiles_per_split >= 1 && workspace)),
+                "mixed_attention_q16: %d splits of %d tiles", splits, tiles_per_split);
     TFF_REQUIRE(G > 0 && H % G == 0 && bt_width > 0 && tff_mixed_attention_q16_supported(H, D, page_size, mix != nullptr),
                 "mixed_attention_q16: %d heads of %d on %d kv heads, pages of %d", H, D, G, page_size);
     TFF_REQUIRE(!bias || bias_rows > 0, "mixed_attention_q16: a bias table without rows");
@@ -632,10 +657,13 @@ TFF_API int tff_mixed_attention_q16(const void* q, const void* k_cache, const vo
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = q16_lds_bytes(H, mix != nullptr);
     const int hpw = (H + Q16_WAVES - 1) / Q16_WAVES;
+    float* part_o = workspace;
+    float* part_ml = workspace ? workspace + (size_t)T * splits * H * D : nullptr;
 #define Q16_LAUNCH(HPW, EB)                                                                                          \
-    mixed_attention_q16_kernel<HPW, EB><<<items, Q16_THREADS, lds, s>>>(                                            \
+    mixed_attention_q16_kernel<HPW, EB><<<dim3(items, splits), Q16_THREADS, lds, s>>>(                              \
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_width, token_req,       \
-        positions, work, bias, bias_rows, mix, scale, cap, window, keep_first, sink, (bf16_t*)out, H, G, page_size)
+        positions, work, bias, bias_rows, mix, scale, cap, window, keep_first, sink, (bf16_t*)out, H, G, page_size, \
+        tiles_per_split, part_o, part_ml)
 #define Q16_BY_EB(HPW)                  \
     do {                                \
         if (D == 32) Q16_LAUNCH(HPW, 2); \
@@ -647,7 +675,10 @@ TFF_API int tff_mixed_attention_q16(const void* q, const void* k_cache, const vo
     else Q16_BY_EB(4);
 #undef Q16_BY_EB
 #undef Q16_LAUNCH
-    return tff_check_launch("mixed_attention_q16");
+    int rc = tff_check_launch("mixed_attention_q16");
+    if (rc || splits <= 1) return rc;
+    mixed_attention_merge_kernel<bf16_t><<<T * H, 64, 0, s>>>(part_o, part_ml, splits, sink, (bf16_t*)out, H, D);
+    return tff_check_launch("mixed_attention_merge");
 }
 
 static size_t ma_lds_bytes(int H, int D, bool mix) {

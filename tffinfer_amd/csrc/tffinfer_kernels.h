@@ -328,13 +328,14 @@ TFF_API int tff_mixed_attention(const void* q, const void* k_cache, const void* 
 TFF_API size_t tff_mixed_attention_workspace_bytes(int T, int H, int D, int splits);
 // The same for prompts in bfloat16 (up to 32 heads of 32, 64 or 128, pages of a multiple of 16 tokens): a block per
 // work item (first token of the step, count <= 16; consecutive tokens of one request), the two products on the
-// matrix cores, keys in tiles of 16.
+// matrix cores, keys in tiles of 16; with splits > 1 an item's tiles are dealt to several blocks and merged (workspace of
+// tff_mixed_attention_workspace_bytes(T, H, D, splits) bytes; every token of the step lies in one item).
 TFF_API int tff_mixed_attention_q16_supported(int H, int D, int page_size, int has_mix);
 TFF_API int tff_mixed_attention_q16(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                     int bt_width, const int32_t* token_req, const int32_t* positions, const int32_t* work,
                                     int items, const float* bias, int bias_rows, const float* mix, float scale, float cap,
-                                    int window, int keep_first, int sink, void* out, int H, int G, int D, int page_size,
-                                    tff_stream_t stream);
+                                    int window, int keep_first, int sink, void* out, int T, int H, int G, int D,
+                                    int page_size, int splits, int tiles_per_split, float* workspace, tff_stream_t stream);
 
 TFF_API int tff_swiglu(const void* gu, void* out, int T, int I, int dtype, tff_stream_t stream);
 

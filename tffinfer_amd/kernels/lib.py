@@ -6,7 +6,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 from .build import ensure_built
 
-ABI_VERSION = 29
+ABI_VERSION = 30
 
 
 class KernelLibraryError(RuntimeError):
@@ -66,7 +66,7 @@ _SIGNATURES = {
     "tff_mixed_attention": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _F, _F, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tff_mixed_attention_workspace_bytes": [_I, _I, _I, _I],
     "tff_mixed_attention_q16_supported": [_I, _I, _I, _I],
-    "tff_mixed_attention_q16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _P, _F, _F, _I, _I, _I, _P, _I, _I, _I, _I, _P],
+    "tff_mixed_attention_q16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _P, _F, _F, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "tff_experts_down": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tff_swiglu": [_P, _P, _I, _I, _I, _P],
     "tff_cast": [_P, _I, _P, _I, c_int64, _P],

@@ -1293,6 +1293,8 @@ def qk_bias_norm_store(qk: torch.Tensor, q_bias, k_bias, eps: float, H: int, G: 
 MIXED_ATTENTION_BLOCKS = 512
 #: tokens of a step from which bfloat16 attention runs sixteen queries a block on the matrix cores
 MIXED_ATTENTION_Q16_TOKENS = 64
+#: blocks that kernel's items are spread over where they are fewer (a block a CU)
+MIXED_ATTENTION_Q16_BLOCKS = 256
 
 
 def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: float, softcap: float = 0.0,
@@ -1338,11 +1340,21 @@ def mixed_attention(q: torch.Tensor, H: int, G: int, D: int, kv, batch, scale: f
         if cache is None:
             items = [(t, min(16, cu[r + 1] - t)) for r in range(len(cu) - 1) for t in range(cu[r], cu[r + 1], 16)]
             cache = batch._q16_work = _staging.send(q.device, [np.asarray(items, dtype=np.int32).reshape(-1, 2)])[0]
+        # tiles of 16 keys an item can have at most; where the items are fewer than the CUs, their tiles are dealt
+        # to several blocks
+        reach = min(bt.shape[1] * kv.page_size, getattr(batch, "max_context", 1 << 30))
+        tiles16 = -(-min(keep_first, reach) // 16) + (-(-min(window + 15, reach) // 16) + 1 if window > 0 else -(-reach // 16))
+        parts = max(1, min(tiles16, 8, MIXED_ATTENTION_Q16_BLOCKS // cache.shape[0]))
+        per = -(-tiles16 // parts)
+        parts = -(-tiles16 // per) if parts > 1 else 1
+        ws = None
+        if parts > 1:
+            ws = torch.empty(L.tff_mixed_attention_workspace_bytes(T, H, D, parts) // 4, dtype=torch.float32, device=q.device)
         _lib.check(L.tff_mixed_attention_q16(q.data_ptr(), kv.k_cache.data_ptr(), kv.v_cache.data_ptr(), bt.data_ptr(),
                                              bt.shape[1], batch.token_req.data_ptr(), batch.positions.data_ptr(),
                                              cache.data_ptr(), cache.shape[0], _ptr(bias), rows, _ptr(mix), float(scale),
                                              float(softcap), int(window), int(keep_first), 1 if sink else 0,
-                                             out.data_ptr(), H, G, D, kv.page_size, _stream()))
+                                             out.data_ptr(), T, H, G, D, kv.page_size, parts, per, _ptr(ws), _stream()))
         return out
     # tiles of 64 keys that a token of this step can have at most (what the block tables can hold, or the window
     # and the kept tokens): a size the host knows without reading a position, so a captured step keeps it
