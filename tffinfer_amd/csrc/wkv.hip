@@ -290,8 +290,7 @@ __device__ __forceinline__ float row16_sum(float v) {
 // For long portions (prompts) of heads of 64 or 128 channels (D = 16 * KPT): a token's cost is what bounds a
 // prompt, since its tokens go one after the other.  Here a row of sixteen lanes shares a value channel, each
 // lane KPT key channels, so a token is KPT steps of four instructions and a sum over the row; a block of four
-// waves takes sixteen value channels of a head, D / 16 blocks a head.  A token's r, k, w are read from LDS
-// while the token before it is worked on.
+// waves takes sixteen value channels of a head, D / 16 blocks a head.
 template <int KPT>
 __global__ __launch_bounds__(256) void wkv_recurrence_rows_kernel(
     const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v,
@@ -355,36 +354,21 @@ __global__ __launch_bounds__(256) void wkv_recurrence_rows_kernel(
         const int n = min(C, t1 - base);
         __syncthreads();
         if (base + C < t1) fetch(base + C);
-        float4 nr[Q], nk[Q], nw[Q];
-        float nv;
-        auto read = [&](int c) {
+        // (unrolled by four: only s runs from token to token, one multiply-add an element; the sums over the rows,
+        // the stores and the LDS reads of neighbouring tokens overlap)
+        float* orow = o + (size_t)base * H * D + col + vi;
+#pragma unroll 4
+        for (int c = 0; c < n; ++c) {
             const float4* cr = reinterpret_cast<const float4*>(buf[b][0] + c * D + ks * KPT);
             const float4* ck = reinterpret_cast<const float4*>(buf[b][1] + c * D + ks * KPT);
             const float4* cw = reinterpret_cast<const float4*>(buf[b][2] + c * D + ks * KPT);
-#pragma unroll
-            for (int q = 0; q < Q; ++q) {
-                nr[q] = cr[q];
-                nk[q] = ck[q];
-                nw[q] = cw[q];
-            }
-            nv = bv[b][c * 16 + vl];
-        };
-        read(0);
-        for (int c = 0; c < n; ++c) {
-            float4 cr[Q], ck[Q], cw[Q];
-#pragma unroll
-            for (int q = 0; q < Q; ++q) {
-                cr[q] = nr[q];
-                ck[q] = nk[q];
-                cw[q] = nw[q];
-            }
-            const float vt = nv;
-            if (c + 1 < n) read(c + 1);
+            const float vt = bv[b][c * 16 + vl];
             float acc = 0.f;
 #pragma unroll
             for (int q = 0; q < Q; ++q) {
-                const float rr[4] = {cr[q].x, cr[q].y, cr[q].z, cr[q].w}, kk4[4] = {ck[q].x, ck[q].y, ck[q].z, ck[q].w},
-                            ww[4] = {cw[q].x, cw[q].y, cw[q].z, cw[q].w};
+                const float4 r4 = cr[q], k4 = ck[q], w4 = cw[q];
+                const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk4[4] = {k4.x, k4.y, k4.z, k4.w},
+                            ww[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float kv = kk4[j] * vt;
@@ -393,7 +377,7 @@ __global__ __launch_bounds__(256) void wkv_recurrence_rows_kernel(
                 }
             }
             acc = row16_sum(acc);
-            if (ks == 0) o[(size_t)(base + c) * H * D + col + vi] = acc;
+            if (ks == 0) orow[(size_t)c * H * D] = acc;
         }
         // (the other buffer was last read before this pass's barrier)
         if (base + C < t1) stage(base + C, b ^ 1);
